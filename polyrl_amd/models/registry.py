@@ -96,7 +96,30 @@ MODEL_CONFIGS = {
 }
 
 
-def get_model_config(name: str, override: dict = None) -> DecoderConfig:
+def _hybrid_presets():
+    from .hybrid import bizusun_preset
+    return {
+        # tiny hybrid for CPU unit tests / fast GPU smoke
+        "bizusun-debug": lambda: bizusun_preset(
+            width=64, layers=5, vocab=300, heads=2, experts=4, top=2,
+            window=24,
+            pattern=("general_delta", "latent_attention", "latent_attention",
+                     "mamba2")),
+        # layer sizes of a ~1B-class model (bench: beside llama3-1b)
+        "bizusun-1b": lambda: bizusun_preset(
+            width=2048, layers=16, vocab=128256, heads=32, window=1024),
+    }
+
+
+def get_model_config(name: str, override: dict = None):
+    """Config by registry name, or from a checkpoint folder holding a
+    ``config.json`` (its ``architecture`` picks the family)."""
+    import os
+    if name not in MODEL_CONFIGS and os.path.isdir(name):
+        from .hybrid import read_config_dir
+        return read_config_dir(name)
+    if name not in MODEL_CONFIGS and name in _hybrid_presets():
+        return _hybrid_presets()[name]()
     if name not in MODEL_CONFIGS:
         raise KeyError(f"unknown model {name!r}; known: {sorted(MODEL_CONFIGS)}")
     cfg = MODEL_CONFIGS[name]

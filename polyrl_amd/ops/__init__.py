@@ -13,6 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import ref
+from . import seq  # noqa: F401  (sequence-mixer ops of the hybrid decoders)
 
 _EXT = None
 _EXT_ERR: Optional[str] = None

@@ -1,0 +1,67 @@
+// pybind bindings for the sequence-mixer kernels of the hybrid decoders
+// (module polyrl_amd._hip_seq: builds on its own, so an engine that serves
+// only such a model compiles nothing else).
+#include <torch/extension.h>
+
+void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
+                     torch::Tensor weight, double eps, int64_t mode);
+void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                     torch::Tensor bias, torch::Tensor state,
+                     torch::Tensor cu_q, torch::Tensor state_slot,
+                     torch::Tensor seq_of_tok, bool add_input, bool act_silu);
+void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
+                       torch::Tensor weight, int64_t groups, double eps,
+                       torch::Tensor gate);
+void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
+                      torch::Tensor positions);
+void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
+                         double eps, torch::Tensor positions,
+                         torch::Tensor inv_freq, torch::Tensor cache,
+                         torch::Tensor slot_mapping);
+void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
+                 int64_t mode);
+void seq_gelu_mul_rows(torch::Tensor out, torch::Tensor gate,
+                       torch::Tensor table, torch::Tensor tokens,
+                       int64_t col0);
+void seq_moe_combine(torch::Tensor res, torch::Tensor y, torch::Tensor inv,
+                     double scale);
+void seq_delta_rule(torch::Tensor out, torch::Tensor r, torch::Tensor k,
+                    torch::Tensor v, torch::Tensor w_lin, torch::Tensor a_lin,
+                    torch::Tensor w0, torch::Tensor a_bias,
+                    torch::Tensor state, torch::Tensor cu_q,
+                    torch::Tensor state_slot, double decay_scale,
+                    double key_eps);
+void seq_ssm_scan(torch::Tensor out, torch::Tensor xbc, torch::Tensor dt,
+                  torch::Tensor z, torch::Tensor dt_bias, torch::Tensor a_log,
+                  torch::Tensor d_skip, torch::Tensor state,
+                  torch::Tensor cu_q, torch::Tensor state_slot,
+                  int64_t groups);
+void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
+                          torch::Tensor q_rot, torch::Tensor cache,
+                          torch::Tensor page_table, torch::Tensor seq_of_tok,
+                          torch::Tensor positions, int64_t window,
+                          torch::Tensor sink, double scale);
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("seq_add_rmsnorm", &seq_add_rmsnorm,
+        "fp32 residual add + RMS norm / cast / unit-RMS add");
+  m.def("seq_causal_conv", &seq_causal_conv,
+        "stateful depthwise causal convolution over packed rows");
+  m.def("seq_group_rmsnorm", &seq_group_rmsnorm,
+        "grouped RMS norm with optional sigmoid gate");
+  m.def("seq_rope_partial", &seq_rope_partial,
+        "rotate-half RoPE on a slice of each head, in place");
+  m.def("seq_latent_kv_store", &seq_latent_kv_store,
+        "norm + rotate + write latent cache rows");
+  m.def("seq_act_mul", &seq_act_mul, "silu*b / sigmoid*b / tanh");
+  m.def("seq_gelu_mul_rows", &seq_gelu_mul_rows,
+        "gelu_tanh(gate) * table rows gathered by token");
+  m.def("seq_moe_combine", &seq_moe_combine,
+        "residual += scale * sum of a token's expert rows");
+  m.def("seq_delta_rule", &seq_delta_rule,
+        "generalised delta rule scan (fp32 state, in place)");
+  m.def("seq_ssm_scan", &seq_ssm_scan,
+        "selective state-space scan (fp32 state, in place)");
+  m.def("seq_latent_attention", &seq_latent_attention,
+        "windowed latent attention with softmax sink over paged cache");
+}

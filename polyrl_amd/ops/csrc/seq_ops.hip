@@ -1,0 +1,454 @@
+// Row-wise kernels of the hybrid decoders: fp32-residual add + RMS norms,
+// stateful depthwise causal convolution, grouped RMS norm with an optional
+// sigmoid gate, partial rotary embedding, the latent-cache writer, gated
+// activations, and the expert-output combine.
+//
+// Activations are T (bf16 or fp32); the residual stream, norm statistics,
+// convolution histories and all transcendental math are fp32.  These ops are
+// HBM-bound: one block per row (or a flat grid-stride loop), no LDS staging
+// beyond the block reductions.  Reference semantics: ops/seq_ref.py.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+
+#include "seq_common.h"
+
+// ------------------------------------------------- residual add + RMS norm
+// mode 0: res += y; out = res * rsqrt(mean(res^2)+eps) * w   (w: 1 or D)
+// mode 1: res += y; out = res (cast)                          (no norm)
+// mode 2: res += y * rsqrt(mean(y^2)+eps) * w                 (out unused)
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(
+    T* __restrict__ out, float* __restrict__ res, const T* __restrict__ y,
+    long ldy, const float* __restrict__ w, int wn, int D, float eps,
+    int mode, bool out_is_res) {
+  __shared__ float red[8];
+  const long row = blockIdx.x;
+  float* rr = res + row * D;
+  const T* yr = y ? y + row * ldy : nullptr;
+  float ss = 0.f;
+  if (mode == 2) {
+    for (int i = threadIdx.x; i < D; i += 256) {
+      const float f = ldf(yr + i);
+      ss += f * f;
+    }
+  } else {
+    for (int i = threadIdx.x; i < D; i += 256) {
+      float f = rr[i];
+      if (yr) {
+        f += ldf(yr + i);
+        rr[i] = f;
+      }
+      ss += f * f;
+    }
+  }
+  if (mode == 1) {
+    if (!out_is_res)
+      for (int i = threadIdx.x; i < D; i += 256)
+        stf(out + row * D + i, rr[i]);   // own writes: same thread, same i
+    return;
+  }
+  ss = block_reduce_sum<4>(ss, red);
+  const float inv = rsqrtf(ss / D + eps);
+  if (mode == 0) {
+    for (int i = threadIdx.x; i < D; i += 256)
+      stf(out + row * D + i, rr[i] * inv * w[wn == 1 ? 0 : i]);
+  } else {
+    for (int i = threadIdx.x; i < D; i += 256)
+      rr[i] += ldf(yr + i) * inv * w[wn == 1 ? 0 : i];
+  }
+}
+
+void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
+                     torch::Tensor weight, double eps, int64_t mode) {
+  CHECK_F32(res);
+  TORCH_CHECK(res.dim() == 2);
+  const int D = res.size(1);
+  const long rows = res.size(0);
+  if (rows == 0) return;
+  const bool has_y = y.defined() && y.numel() > 0;
+  if (has_y) {
+    CHECK_ROWS(y);
+    TORCH_CHECK(y.size(0) == rows && y.size(1) == D, "y shape");
+  }
+  TORCH_CHECK(mode != 2 || has_y);
+  const float* w = nullptr;
+  int wn = 0;
+  if (mode != 1) {
+    CHECK_F32(weight);
+    wn = weight.numel();
+    TORCH_CHECK(wn == 1 || wn == D, "norm weight must hold 1 or D numbers");
+    w = weight.data_ptr<float>();
+  }
+  const bool out_is_res = out.data_ptr() == res.data_ptr();
+  if (mode != 2) {
+    TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
+                out.numel() == res.numel());
+  }
+  auto dt = mode == 2 ? y.scalar_type()
+                      : (out_is_res ? (has_y ? y.scalar_type()
+                                             : torch::kFloat32)
+                                    : out.scalar_type());
+  if (has_y) TORCH_CHECK(y.scalar_type() == dt, "y / out dtype mismatch");
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(dt, { hipLaunchKernelGGL((add_rmsnorm_kernel<T>), dim3(rows), dim3(256), 0, stream, 
+      mode == 2 || out_is_res ? nullptr : (T*)out.data_ptr(),
+      res.data_ptr<float>(), has_y ? (const T*)y.data_ptr() : nullptr,
+      has_y ? y.stride(0) : 0, w, wn, D, (float)eps, (int)mode, out_is_res); });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------- stateful causal convolution
+// y_t = sum_j w[c, j] * x_(t - taps + 1 + j) (+ bias) (+ x_t) (silu)
+// history before the portion's first row comes from state[slot] (taps-1, C)
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    T* __restrict__ out, const T* __restrict__ x, long ldx,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slot, const int* __restrict__ seq_of_tok,
+    int C, int taps, bool add_input, bool act_silu) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int b = seq_of_tok[n];
+  const int q0 = cu_q[b];
+  const int t = n - q0;
+  const float* st = state + (long)state_slot[b] * (taps - 1) * C;
+  float acc = bias ? bias[c] : 0.f;
+  float cur = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = t - (taps - 1) + j;
+    const float v = src >= 0 ? ldf(x + (long)(q0 + src) * ldx + c)
+                             : st[(long)(taps - 1 + src) * C + c];
+    acc += w[(long)c * taps + j] * v;
+    cur = v;
+  }
+  if (add_input) acc += cur;
+  if (act_silu) acc = siluf_acc(acc);
+  stf(out + (long)n * C + c, acc);
+}
+
+// new history = last taps-1 rows of [old history ; portion].  Ascending
+// order is safe in place: row i reads old row i+L (L >= 1), never a row
+// already overwritten; each thread owns one channel column.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(
+    float* __restrict__ state, const T* __restrict__ x, long ldx,
+    const int* __restrict__ cu_q, const int* __restrict__ state_slot, int C,
+    int taps) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int q0 = cu_q[b];
+  const int L = cu_q[b + 1] - q0;
+  if (L <= 0) return;
+  float* st = state + (long)state_slot[b] * (taps - 1) * C;
+  for (int i = 0; i < taps - 1; ++i) {
+    const int h = L + i;                      // index into [old ; portion]
+    st[(long)i * C + c] = h < taps - 1
+                              ? st[(long)h * C + c]
+                              : ldf(x + (long)(q0 + h - (taps - 1)) * ldx + c);
+  }
+}
+
+void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                     torch::Tensor bias, torch::Tensor state,
+                     torch::Tensor cu_q, torch::Tensor state_slot,
+                     torch::Tensor seq_of_tok, bool add_input, bool act_silu) {
+  CHECK_ROWS(x);
+  CHECK_F32(w);
+  CHECK_F32(state);
+  CHECK_I32(cu_q);
+  CHECK_I32(state_slot);
+  CHECK_I32(seq_of_tok);
+  const int N = x.size(0), C = w.size(0), taps = w.size(1);
+  TORCH_CHECK(x.size(1) == C && out.is_contiguous() && out.size(0) == N &&
+              out.size(1) == C && out.scalar_type() == x.scalar_type());
+  TORCH_CHECK(taps >= 1 && state.dim() == 3 && state.size(1) == taps - 1 &&
+              state.size(2) == C, "state must be (slots, taps-1, C)");
+  TORCH_CHECK(seq_of_tok.numel() == N && cu_q.numel() == state_slot.numel() + 1);
+  const float* bp = nullptr;
+  if (bias.defined() && bias.numel() > 0) {
+    CHECK_F32(bias);
+    TORCH_CHECK(bias.numel() == C);
+    bp = bias.data_ptr<float>();
+  }
+  const int B = state_slot.numel();
+  auto stream = at::hip::getCurrentHIPStream();
+  const int cb = (C + 255) / 256;
+  SEQ_DISPATCH_T(x.scalar_type(), {
+    hipLaunchKernelGGL((causal_conv_kernel<T>), dim3(N, cb), dim3(256), 0, stream, 
+        (T*)out.data_ptr(), (const T*)x.data_ptr(), x.stride(0),
+        w.data_ptr<float>(), bp, state.data_ptr<float>(),
+        cu_q.data_ptr<int>(), state_slot.data_ptr<int>(),
+        seq_of_tok.data_ptr<int>(), C, taps, add_input, act_silu);
+    if (taps > 1)
+      hipLaunchKernelGGL((conv_state_kernel<T>), dim3(B, cb), dim3(256), 0, stream, 
+          state.data_ptr<float>(), (const T*)x.data_ptr(), x.stride(0),
+          cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), C, taps);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------ grouped RMS norm (+gate)
+// out = y / rms_group(y) * w * (gate ? sigmoid(gate) : 1); one wave per
+// (row, group), groups of a row round-robin over the block's 4 waves.
+template <typename T>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(
+    T* __restrict__ out, const float* __restrict__ y,
+    const float* __restrict__ w, const T* __restrict__ gate, long ldg, int D,
+    int groups, float eps) {
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wid = threadIdx.x >> 6;
+  const int gs = D / groups;
+  for (int g = wid; g < groups; g += 4) {
+    const float* yr = y + row * D + (long)g * gs;
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += 64) ss += yr[i] * yr[i];
+    ss = wave_reduce_sum(ss);
+    const float inv = rsqrtf(ss / gs + eps);
+    for (int i = lane; i < gs; i += 64) {
+      const int c = g * gs + i;
+      float v = yr[i] * inv * w[c];
+      if (gate) v *= sigmoidf_acc(ldf(gate + row * ldg + c));
+      stf(out + row * D + c, v);
+    }
+  }
+}
+
+void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
+                       torch::Tensor weight, int64_t groups, double eps,
+                       torch::Tensor gate) {
+  CHECK_F32(y);
+  CHECK_F32(weight);
+  TORCH_CHECK(y.dim() == 2 && out.is_contiguous() && out.sizes() == y.sizes());
+  const int D = y.size(1);
+  TORCH_CHECK(groups >= 1 && D % groups == 0 && weight.numel() == D);
+  const bool has_g = gate.defined() && gate.numel() > 0;
+  if (has_g) {
+    CHECK_ROWS(gate);
+    TORCH_CHECK(gate.size(0) == y.size(0) && gate.size(1) == D &&
+                gate.scalar_type() == out.scalar_type());
+  }
+  if (y.size(0) == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(out.scalar_type(), { hipLaunchKernelGGL((group_rmsnorm_kernel<T>), dim3(y.size(0)), dim3(256), 0, stream, 
+      (T*)out.data_ptr(), y.data_ptr<float>(), weight.data_ptr<float>(),
+      has_g ? (const T*)gate.data_ptr() : nullptr, has_g ? gate.stride(0) : 0,
+      D, (int)groups, (float)eps); });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------- partial rotary (q)
+// q (N, H, Dh) with token stride ldn: rotate the pair (off+i, off+i+half)
+// by angle fp32(pos) * inv_freq[i].
+template <typename T>
+__global__ void rope_partial_kernel(T* __restrict__ q, long ldn, int H, int Dh,
+                                    int off, const float* __restrict__ inv_freq,
+                                    int half, const int* __restrict__ pos,
+                                    long total) {
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int i = idx % half;
+  const int h = (idx / half) % H;
+  const long n = idx / ((long)half * H);
+  const float ang = (float)pos[n] * inv_freq[i];
+  const float c = cosf(ang), s = sinf(ang);
+  T* p = q + n * ldn + (long)h * Dh + off + i;
+  const float a = ldf(p), b = ldf(p + half);
+  stf(p, a * c - b * s);
+  stf(p + half, b * c + a * s);
+}
+
+void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
+                      torch::Tensor positions) {
+  CHECK_F32(inv_freq);
+  CHECK_I32(positions);
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.stride(2) == 1 &&
+              q.stride(1) == q.size(2), "q must be (N, H, Dh), heads packed");
+  const int half = inv_freq.numel();
+  TORCH_CHECK(offset >= 0 && offset + 2 * half <= q.size(2));
+  TORCH_CHECK(positions.numel() == q.size(0));
+  const long total = (long)q.size(0) * q.size(1) * half;
+  if (total == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(q.scalar_type(), { hipLaunchKernelGGL((rope_partial_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, 
+      (T*)q.data_ptr(), q.stride(0), (int)q.size(1), (int)q.size(2),
+      (int)offset, inv_freq.data_ptr<float>(), half,
+      positions.data_ptr<int>(), total); });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------------ latent cache store
+// one wave per token: RMS-norm the latent (first R columns) times norm_w,
+// rotate the first 2*half columns of the key part, write the cache row.
+template <typename T>
+__global__ __launch_bounds__(64) void latent_store_kernel(
+    const T* __restrict__ dkv, long ld, int R, int rd,
+    const float* __restrict__ norm_w, float eps, const int* __restrict__ pos,
+    const float* __restrict__ inv_freq, int half, T* __restrict__ cache,
+    const int* __restrict__ slot_mapping) {
+  const long n = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int slot = slot_mapping[n];
+  if (slot < 0) return;
+  const T* src = dkv + n * ld;
+  T* dst = cache + (long)slot * (R + rd);
+  float ss = 0.f;
+  for (int i = lane; i < R; i += 64) {
+    const float f = ldf(src + i);
+    ss += f * f;
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = rsqrtf(ss / R + eps);
+  for (int i = lane; i < R; i += 64) stf(dst + i, ldf(src + i) * inv * norm_w[i]);
+  const float p = (float)pos[n];
+  for (int i = lane; i < half; i += 64) {
+    const float ang = p * inv_freq[i];
+    const float c = cosf(ang), s = sinf(ang);
+    const float a = ldf(src + R + i), b = ldf(src + R + i + half);
+    stf(dst + R + i, a * c - b * s);
+    stf(dst + R + i + half, b * c + a * s);
+  }
+  for (int i = 2 * half + lane; i < rd; i += 64) stf(dst + R + i, ldf(src + R + i));
+}
+
+void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
+                         double eps, torch::Tensor positions,
+                         torch::Tensor inv_freq, torch::Tensor cache,
+                         torch::Tensor slot_mapping) {
+  CHECK_ROWS(dkv);
+  CHECK_F32(norm_w);
+  CHECK_F32(inv_freq);
+  CHECK_I32(positions);
+  CHECK_I32(slot_mapping);
+  const int N = dkv.size(0), row = dkv.size(1);
+  const int half = inv_freq.numel();
+  TORCH_CHECK(rank > 0 && rank <= row && norm_w.numel() == rank);
+  TORCH_CHECK(2 * half <= row - rank);
+  TORCH_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 &&
+              cache.size(2) == row && cache.scalar_type() == dkv.scalar_type());
+  TORCH_CHECK(positions.numel() == N && slot_mapping.numel() == N);
+  if (N == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(dkv.scalar_type(), { hipLaunchKernelGGL((latent_store_kernel<T>), dim3(N), dim3(64), 0, stream, 
+      (const T*)dkv.data_ptr(), dkv.stride(0), (int)rank, (int)(row - rank),
+      norm_w.data_ptr<float>(), (float)eps, positions.data_ptr<int>(),
+      inv_freq.data_ptr<float>(), half, (T*)cache.data_ptr(),
+      slot_mapping.data_ptr<int>()); });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------------- gated activations
+// mode 0: silu(a) * b   mode 1: sigmoid(a) * b   mode 2: tanh(a)
+template <typename T>
+__global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
+                               long lda, const T* __restrict__ b, long ldb,
+                               long rows, int cols, int mode) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long stride = (long)gridDim.x * blockDim.x;
+  const long n = rows * cols;
+  for (; i < n; i += stride) {
+    const long r = i / cols;
+    const int c = i % cols;
+    const float av = ldf(a + r * lda + c);
+    float v;
+    if (mode == 2) {
+      v = tanhf(av);
+    } else {
+      const float bv = ldf(b + r * ldb + c);
+      v = (mode == 0 ? siluf_acc(av) : sigmoidf_acc(av)) * bv;
+    }
+    stf(out + i, v);
+  }
+}
+
+void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
+                 int64_t mode) {
+  CHECK_ROWS(a);
+  CHECK_ROWS(b);
+  TORCH_CHECK(a.sizes() == b.sizes() && out.is_contiguous() &&
+              out.sizes() == a.sizes() &&
+              a.scalar_type() == b.scalar_type() &&
+              out.scalar_type() == a.scalar_type());
+  const long rows = a.size(0);
+  const int cols = a.size(1);
+  if (rows * cols == 0) return;
+  const long nblk = std::min<long>((rows * cols + 255) / 256, MAX_RESIDENT_BLOCKS * 4);
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(a.scalar_type(), { hipLaunchKernelGGL((act_mul_kernel<T>), dim3(nblk), dim3(256), 0, stream, 
+      (T*)out.data_ptr(), (const T*)a.data_ptr(), a.stride(0),
+      (const T*)b.data_ptr(), b.stride(0), rows, cols, (int)mode); });
+  HIP_CHECK_KERNEL();
+}
+
+// out = gelu_tanh(gate) * table[tokens[n], col0 + c]
+template <typename T>
+__global__ void gelu_mul_rows_kernel(T* __restrict__ out,
+                                     const T* __restrict__ gate, long ldg,
+                                     const T* __restrict__ table, long ldt,
+                                     const long* __restrict__ tokens, int col0,
+                                     long rows, int cols) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * cols) return;
+  const long r = i / cols;
+  const int c = i % cols;
+  const float z = ldf(gate + r * ldg + c);
+  const float e = ldf(table + tokens[r] * ldt + col0 + c);
+  stf(out + i, gelu_tanhf_acc(z) * e);
+}
+
+void seq_gelu_mul_rows(torch::Tensor out, torch::Tensor gate,
+                       torch::Tensor table, torch::Tensor tokens,
+                       int64_t col0) {
+  CHECK_ROWS(gate);
+  CHECK_ROWS(table);
+  TORCH_CHECK(tokens.is_cuda() && tokens.dtype() == torch::kInt64 &&
+              tokens.is_contiguous() && tokens.numel() == gate.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == gate.sizes() &&
+              table.scalar_type() == gate.scalar_type() &&
+              out.scalar_type() == gate.scalar_type());
+  TORCH_CHECK(col0 >= 0 && col0 + gate.size(1) <= table.size(1));
+  const long n = gate.numel();
+  if (n == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(gate.scalar_type(), { hipLaunchKernelGGL((gelu_mul_rows_kernel<T>), dim3((n + 255) / 256), dim3(256), 0, stream, 
+      (T*)out.data_ptr(), (const T*)gate.data_ptr(), gate.stride(0),
+      (const T*)table.data_ptr(), table.stride(0),
+      (const long*)tokens.data_ptr<int64_t>(), (int)col0, gate.size(0),
+      (int)gate.size(1)); });
+  HIP_CHECK_KERNEL();
+}
+
+// res[n, d] += scale * sum_k y[inv[n, k], d]
+template <typename T>
+__global__ void moe_combine_kernel(float* __restrict__ res,
+                                   const T* __restrict__ y,
+                                   const int* __restrict__ inv, int top,
+                                   float scale, long rows, int D) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * D) return;
+  const long n = i / D;
+  const int d = i % D;
+  float acc = 0.f;
+  for (int k = 0; k < top; ++k) acc += ldf(y + (long)inv[n * top + k] * D + d);
+  res[i] += scale * acc;
+}
+
+void seq_moe_combine(torch::Tensor res, torch::Tensor y, torch::Tensor inv,
+                     double scale) {
+  CHECK_F32(res);
+  CHECK_I32(inv);
+  TORCH_CHECK(res.dim() == 2 && inv.dim() == 2 && inv.size(0) == res.size(0));
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.dim() == 2 &&
+              y.size(1) == res.size(1) &&
+              y.size(0) == inv.size(0) * inv.size(1));
+  const long n = res.numel();
+  if (n == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(y.scalar_type(), { hipLaunchKernelGGL((moe_combine_kernel<T>), dim3((n + 255) / 256), dim3(256), 0, stream, 
+      res.data_ptr<float>(), (const T*)y.data_ptr(), inv.data_ptr<int>(),
+      (int)inv.size(1), (float)scale, res.size(0), (int)res.size(1)); });
+  HIP_CHECK_KERNEL();
+}

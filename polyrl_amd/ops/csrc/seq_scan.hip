@@ -1,0 +1,310 @@
+// Recurrent scans of the hybrid decoders, one launch for prefill portions
+// and decode tokens alike (a decode token is a portion of length 1):
+//
+//   delta rule : S <- diag(w) S - (a*u)(u^T S) + k v^T ,  o = S^T r
+//   state space: S <- exp(-exp(A) dt) S + dt B x^T     ,  y = S^T C + D x
+//
+// State columns are independent in both recurrences, so the state matrix
+// (rows = key/state channel, columns = value channel) is spread over a wave
+// as 16 columns x 4 row-groups: a lane keeps RPL = rows/4 state entries of
+// one column in VGPRs for the whole portion, the two per-token reductions
+// over rows (u^T S and S^T r, or S^T C) are two xor-shuffles inside the
+// 4-lane group, and a wave never synchronises with another.  The grid is
+// (sequence, head, 64-column block); HBM traffic is the state once in and
+// once out per portion plus the token inputs.  Inputs of token t+1 are
+// loaded before the arithmetic of token t so the dependent chain per token
+// is the VALU work only.  All state math is fp32 for bf16 or fp32 inputs.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+
+#include "seq_common.h"
+
+constexpr int RG = 4;            // lanes sharing one column (row groups)
+constexpr int COLS_PER_WAVE = 16;
+
+// ------------------------------------------------------------- delta rule
+template <typename T, int RPL>
+struct DeltaIn {
+  float r[RPL], k[RPL], wl[RPL], al[RPL];
+  float v;
+};
+
+template <typename T, int RPL>
+DEV_INLINE void delta_load(DeltaIn<T, RPL>& in, const T* r, const T* k,
+                           const T* v, const T* wl, const T* al, long ldr,
+                           long ldk, long ldv, long ldw, long lda, long n,
+                           int hoff_k, int row0, int Dk, int vcol, bool colok) {
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    const bool ok = row < Dk;
+    in.r[i] = ok ? ldf(r + n * ldr + hoff_k + row) : 0.f;
+    in.k[i] = ok ? ldf(k + n * ldk + hoff_k + row) : 0.f;
+    in.wl[i] = ok ? ldf(wl + n * ldw + hoff_k + row) : 0.f;
+    in.al[i] = ok ? ldf(al + n * lda + hoff_k + row) : 0.f;
+  }
+  in.v = colok ? ldf(v + n * ldv + vcol) : 0.f;
+}
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(256) void delta_rule_kernel(
+    float* __restrict__ out,            // (N, H*Dv) fp32, un-normalised o
+    const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ wl, const T* __restrict__ al, long ldr, long ldk,
+    long ldv, long ldw, long lda, const float* __restrict__ w0,
+    const float* __restrict__ a_bias, float* __restrict__ state,
+    const int* __restrict__ cu_q, const int* __restrict__ state_slot, int H,
+    int Dk, int Dv, float decay_scale, float key_eps) {
+  const int cblocks = (Dv + 63) / 64;
+  const int b = blockIdx.x / (H * cblocks);
+  const int h = (blockIdx.x / cblocks) % H;
+  const int cb = blockIdx.x % cblocks;
+  const int lane = threadIdx.x & 63;
+  const int wid = threadIdx.x >> 6;
+  const int col = cb * 64 + wid * COLS_PER_WAVE + lane / RG;
+  const int rg = lane % RG;
+  const int row0 = rg * RPL;
+  const bool colok = col < Dv;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (q1 <= q0) return;
+  // a whole wave past the last column has nothing to do (wave-uniform)
+  if (cb * 64 + wid * COLS_PER_WAVE >= Dv) return;
+
+  float* S = state + (((long)state_slot[b] * H + h) * Dk) * Dv;
+  float s[RPL], w0r[RPL], abr[RPL];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    const bool ok = colok && row < Dk;
+    s[i] = ok ? S[(long)row * Dv + col] : 0.f;
+    w0r[i] = row < Dk ? w0[h * Dk + row] : 0.f;
+    abr[i] = row < Dk ? a_bias[h * Dk + row] : 0.f;
+  }
+  const int hoff_k = h * Dk;
+  const int vcol = h * Dv + col;
+
+  DeltaIn<T, RPL> cur, nxt;
+  delta_load<T, RPL>(cur, r, k, v, wl, al, ldr, ldk, ldv, ldw, lda, q0,
+                     hoff_k, row0, Dk, vcol, colok);
+  for (int n = q0; n < q1; ++n) {
+    if (n + 1 < q1)
+      delta_load<T, RPL>(nxt, r, k, v, wl, al, ldr, ldk, ldv, ldw, lda, n + 1,
+                         hoff_k, row0, Dk, vcol, colok);
+    // unit key: |k|^2 over the head's Dk rows = sum over the 4 row groups
+    float kk = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) kk += cur.k[i] * cur.k[i];
+    kk = lanegroup_sum<RG>(kk);
+    const float kinv = rsqrtf(kk + key_eps);
+    float p = 0.f;
+    float u[RPL];
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      u[i] = cur.k[i] * kinv;
+      p += u[i] * s[i];
+    }
+    p = lanegroup_sum<RG>(p);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      const float dec = expf(-decay_scale * sigmoidf_acc(cur.wl[i] + w0r[i]));
+      const float rem = sigmoidf_acc(cur.al[i] + abr[i]);
+      s[i] = dec * s[i] - rem * u[i] * p + cur.k[i] * cur.v;
+      o += s[i] * cur.r[i];
+    }
+    o = lanegroup_sum<RG>(o);
+    if (colok && rg == 0) out[(long)n * H * Dv + vcol] = o;
+    cur = nxt;
+  }
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    if (colok && row < Dk) S[(long)row * Dv + col] = s[i];
+  }
+}
+
+#define DELTA_LAUNCH(RPLV)                                                   \
+  hipLaunchKernelGGL((delta_rule_kernel<T, RPLV>), dim3(grid), dim3(256), 0, stream,           \
+      out.data_ptr<float>(), (const T*)r.data_ptr(), (const T*)k.data_ptr(), \
+      (const T*)v.data_ptr(), (const T*)w_lin.data_ptr(),                    \
+      (const T*)a_lin.data_ptr(), r.stride(0), k.stride(0), v.stride(0),     \
+      w_lin.stride(0), a_lin.stride(0), w0.data_ptr<float>(),                \
+      a_bias.data_ptr<float>(), state.data_ptr<float>(),                     \
+      cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Dk, Dv,           \
+      (float)decay_scale, (float)key_eps)
+
+void seq_delta_rule(torch::Tensor out, torch::Tensor r, torch::Tensor k,
+                    torch::Tensor v, torch::Tensor w_lin, torch::Tensor a_lin,
+                    torch::Tensor w0, torch::Tensor a_bias,
+                    torch::Tensor state, torch::Tensor cu_q,
+                    torch::Tensor state_slot, double decay_scale,
+                    double key_eps) {
+  CHECK_ROWS(r); CHECK_ROWS(k); CHECK_ROWS(v); CHECK_ROWS(w_lin);
+  CHECK_ROWS(a_lin);
+  CHECK_F32(w0); CHECK_F32(a_bias); CHECK_F32(state); CHECK_F32(out);
+  CHECK_I32(cu_q); CHECK_I32(state_slot);
+  TORCH_CHECK(state.dim() == 4);
+  const int H = state.size(1), Dk = state.size(2), Dv = state.size(3);
+  const long N = r.size(0);
+  TORCH_CHECK(r.size(1) == H * Dk && k.size(1) == H * Dk &&
+              w_lin.size(1) == H * Dk && a_lin.size(1) == H * Dk &&
+              v.size(1) == H * Dv, "delta rule operand widths");
+  TORCH_CHECK(k.size(0) == N && v.size(0) == N && w_lin.size(0) == N &&
+              a_lin.size(0) == N && out.size(0) == N &&
+              out.size(1) == H * Dv);
+  TORCH_CHECK(w0.numel() == H * Dk && a_bias.numel() == H * Dk);
+  auto dt = r.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt &&
+              w_lin.scalar_type() == dt && a_lin.scalar_type() == dt);
+  TORCH_CHECK(Dk <= 256, "delta rule: key dim above 256 not supported");
+  const int B = state_slot.numel();
+  TORCH_CHECK(cu_q.numel() == B + 1);
+  if (N == 0 || B == 0) return;
+  const int grid = B * H * ((Dv + 63) / 64);
+  const int rpl = (Dk + RG - 1) / RG;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(dt, {
+    if (rpl <= 4) DELTA_LAUNCH(4);
+    else if (rpl <= 8) DELTA_LAUNCH(8);
+    else if (rpl <= 16) DELTA_LAUNCH(16);
+    else if (rpl <= 32) DELTA_LAUNCH(32);
+    else DELTA_LAUNCH(64);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------------------ state space
+template <int RPL>
+struct SsmIn {
+  float Bv[RPL], Cv[RPL];
+  float x, dt, z;
+};
+
+template <typename T, int RPL>
+DEV_INLINE void ssm_load(SsmIn<RPL>& in, const T* xbc, long ldx, const T* dt,
+                         long ldd, const T* z, long ldz, long n, int xcol,
+                         int boff, int coff, int row0, int Ns, int h,
+                         bool colok) {
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    const bool ok = row < Ns;
+    in.Bv[i] = ok ? ldf(xbc + n * ldx + boff + row) : 0.f;
+    in.Cv[i] = ok ? ldf(xbc + n * ldx + coff + row) : 0.f;
+  }
+  in.x = colok ? ldf(xbc + n * ldx + xcol) : 0.f;
+  in.z = colok ? ldf(z + n * ldz + xcol) : 0.f;
+  in.dt = ldf(dt + n * ldd + h);
+}
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(
+    float* __restrict__ out,            // (N, H*P) fp32: y * silu(z)
+    const T* __restrict__ xbc, long ldx, const T* __restrict__ dt, long ldd,
+    const T* __restrict__ z, long ldz, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, const float* __restrict__ d_skip,
+    float* __restrict__ state, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slot, int H, int Ns, int P, int G) {
+  const int cblocks = (P + 63) / 64;
+  const int b = blockIdx.x / (H * cblocks);
+  const int h = (blockIdx.x / cblocks) % H;
+  const int cb = blockIdx.x % cblocks;
+  const int lane = threadIdx.x & 63;
+  const int wid = threadIdx.x >> 6;
+  const int col = cb * 64 + wid * COLS_PER_WAVE + lane / RG;
+  const int rg = lane % RG;
+  const int row0 = rg * RPL;
+  const bool colok = col < P;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (q1 <= q0) return;
+  if (cb * 64 + wid * COLS_PER_WAVE >= P) return;
+
+  const int inner = H * P;
+  const int g = h / (H / G);
+  const int boff = inner + g * Ns;
+  const int coff = inner + G * Ns + g * Ns;
+  const int xcol = h * P + col;
+  float* S = state + (((long)state_slot[b] * H + h) * Ns) * P;
+  float s[RPL];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    s[i] = (colok && row < Ns) ? S[(long)row * P + col] : 0.f;
+  }
+  const float A = expf(a_log[h]);
+  const float Dh = d_skip[h];
+  const float dtb = dt_bias[h];
+
+  SsmIn<RPL> cur, nxt;
+  ssm_load<T, RPL>(cur, xbc, ldx, dt, ldd, z, ldz, q0, xcol, boff, coff, row0,
+                   Ns, h, colok);
+  for (int n = q0; n < q1; ++n) {
+    if (n + 1 < q1)
+      ssm_load<T, RPL>(nxt, xbc, ldx, dt, ldd, z, ldz, n + 1, xcol, boff,
+                       coff, row0, Ns, h, colok);
+    const float step = softplusf_acc(cur.dt + dtb);
+    const float dec = expf(-A * step);
+    const float sx = step * cur.x;
+    float y = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      s[i] = dec * s[i] + cur.Bv[i] * sx;
+      y += s[i] * cur.Cv[i];
+    }
+    y = lanegroup_sum<RG>(y);
+    if (colok && rg == 0)
+      out[(long)n * inner + xcol] = (y + Dh * cur.x) * siluf_acc(cur.z);
+    cur = nxt;
+  }
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    if (colok && row < Ns) S[(long)row * P + col] = s[i];
+  }
+}
+
+#define SSM_LAUNCH(RPLV)                                                     \
+  hipLaunchKernelGGL((ssm_scan_kernel<T, RPLV>), dim3(grid), dim3(256), 0, stream,             \
+      out.data_ptr<float>(), (const T*)xbc.data_ptr(), xbc.stride(0),        \
+      (const T*)dt.data_ptr(), dt.stride(0), (const T*)z.data_ptr(),         \
+      z.stride(0), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),       \
+      d_skip.data_ptr<float>(), state.data_ptr<float>(),                     \
+      cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Ns, P, (int)groups)
+
+void seq_ssm_scan(torch::Tensor out, torch::Tensor xbc, torch::Tensor dt,
+                  torch::Tensor z, torch::Tensor dt_bias, torch::Tensor a_log,
+                  torch::Tensor d_skip, torch::Tensor state,
+                  torch::Tensor cu_q, torch::Tensor state_slot,
+                  int64_t groups) {
+  CHECK_ROWS(xbc); CHECK_ROWS(dt); CHECK_ROWS(z);
+  CHECK_F32(dt_bias); CHECK_F32(a_log); CHECK_F32(d_skip); CHECK_F32(state);
+  CHECK_F32(out);
+  CHECK_I32(cu_q); CHECK_I32(state_slot);
+  TORCH_CHECK(state.dim() == 4);
+  const int H = state.size(1), Ns = state.size(2), P = state.size(3);
+  const long N = xbc.size(0);
+  TORCH_CHECK(groups >= 1 && H % groups == 0);
+  TORCH_CHECK(xbc.size(1) == H * P + 2 * groups * Ns && dt.size(1) == H &&
+              z.size(1) == H * P && dt.size(0) == N && z.size(0) == N &&
+              out.size(0) == N && out.size(1) == H * P,
+              "state-space operand widths");
+  TORCH_CHECK(dt_bias.numel() == H && a_log.numel() == H &&
+              d_skip.numel() == H);
+  auto ty = xbc.scalar_type();
+  TORCH_CHECK(dt.scalar_type() == ty && z.scalar_type() == ty);
+  TORCH_CHECK(Ns <= 256, "state size above 256 not supported");
+  const int B = state_slot.numel();
+  TORCH_CHECK(cu_q.numel() == B + 1);
+  if (N == 0 || B == 0) return;
+  const int grid = B * H * ((P + 63) / 64);
+  const int rpl = (Ns + RG - 1) / RG;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(ty, {
+    if (rpl <= 4) SSM_LAUNCH(4);
+    else if (rpl <= 8) SSM_LAUNCH(8);
+    else if (rpl <= 16) SSM_LAUNCH(16);
+    else if (rpl <= 32) SSM_LAUNCH(32);
+    else SSM_LAUNCH(64);
+  });
+  HIP_CHECK_KERNEL();
+}

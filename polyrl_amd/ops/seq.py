@@ -1,0 +1,245 @@
+"""Sequence-mixer ops for hybrid decoders: fp32-residual norms, stateful
+causal convolutions, the generalised delta rule, the selective state-space
+scan, and windowed latent attention with a softmax sink.
+
+Same policy as the rest of ``polyrl_amd.ops``: on a HIP device the in-tree
+extension is REQUIRED (csrc/seq_*.hip, templated on the activation type:
+bf16 or fp32); CPU tensors run the PyTorch forms in seq_ref.py.  What the
+recurrences consume (decays, step sizes, gates, unit keys, states) and all
+norms, scores and softmax weights are fp32 inside the kernels for either
+activation type.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import seq_ref as R
+
+
+_SEQ_EXT = None
+_SEQ_ERR: Optional[str] = None
+try:
+    from polyrl_amd import _hip_seq as _SEQ_EXT  # type: ignore
+except Exception as e:  # pragma: no cover - import-environment dependent
+    _SEQ_ERR = repr(e)
+
+
+def seq_extension_loaded() -> bool:
+    return _SEQ_EXT is not None
+
+
+def _ext():
+    if _SEQ_EXT is None:
+        raise RuntimeError(
+            "polyrl_amd._hip_seq extension is required on GPU but failed to "
+            f"load ({_SEQ_ERR}). Build it in-tree: "
+            "PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace")
+    return _SEQ_EXT
+
+
+def add_rmsnorm_f32res(res: torch.Tensor, y: Optional[torch.Tensor],
+                       weight: torch.Tensor, eps: float,
+                       out_dtype: torch.dtype) -> torch.Tensor:
+    """res (N, D) fp32 += y in place, then RMS-norm(res) * weight -> out_dtype.
+    ``weight`` holds one number (for all coordinates) or D."""
+    if res.is_cuda:
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
+                               weight, eps, 0)
+        return out
+    return R.add_rmsnorm_f32res(res, y, weight, eps, out_dtype)
+
+
+def residual_add_cast(res: torch.Tensor, y: Optional[torch.Tensor],
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """res += y in place; returns res in out_dtype (res itself for fp32)."""
+    if res.is_cuda:
+        if y is None and out_dtype == torch.float32:
+            return res
+        out = res if out_dtype == torch.float32 else \
+            torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
+                               torch.Tensor(), 0.0, 1)
+        return out
+    return R.residual_add_cast(res, y, out_dtype)
+
+
+def add_scaled_unit_rms(res: torch.Tensor, y: torch.Tensor,
+                        weight: torch.Tensor, eps: float) -> None:
+    """res += y / rms(y) * weight, in place (weight (D,) fp32)."""
+    if res.is_cuda:
+        _ext().seq_add_rmsnorm(res, res, y, weight, eps, 2)
+        return
+    R.add_scaled_unit_rms(res, y, weight, eps)
+
+
+def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,
+                      add_input: bool, act_silu: bool,
+                      out_dtype) -> torch.Tensor:
+    """Depthwise causal convolution over each sequence's rows with the last
+    taps-1 inputs carried in ``state`` (slots, taps-1, C) fp32.
+    y_t = sum_j w[:, j] x_(t-taps+1+j) [+ bias] [+ x_t], optional SiLU.
+    ``x`` may be a column slice (row-strided view)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], w.shape[0], dtype=out_dtype,
+                          device=x.device)
+        if x.shape[0]:
+            _ext().seq_causal_conv(out, x, w,
+                                   bias if bias is not None else torch.Tensor(),
+                                   state, cu_q, state_slot, seq_of_tok,
+                                   add_input, act_silu)
+        return out
+    return R.causal_conv_state(x, w, bias, state, cu_q, state_slot,
+                               seq_of_tok, add_input, act_silu, out_dtype)
+
+
+def delta_rule(r, k, v, w_lin, a_lin, g, w0, a_bias, norm_w, state, cu_q,
+               state_slot, decay_scale: float, key_eps: float, eps: float,
+               out_dtype) -> torch.Tensor:
+    """Generalised delta rule over packed rows; ``state`` (slots, H, Dk, Dv)
+    fp32 in place.  Per head: w = exp(-decay_scale*sigmoid(w_lin + w0)),
+    a = sigmoid(a_lin + a_bias), u = k/sqrt(|k|^2+key_eps),
+    S <- diag(w) S - (a*u)(u^T S) + k v^T, o = S^T r; returns
+    o/rms_head(o) * norm_w * sigmoid(g).  Inputs may be column slices."""
+    if r.is_cuda:
+        slots, H, Dk, Dv = state.shape
+        out = torch.empty(r.shape[0], H * Dv, dtype=out_dtype, device=r.device)
+        if r.shape[0]:
+            o = torch.empty(r.shape[0], H * Dv, dtype=torch.float32,
+                            device=r.device)
+            _ext().seq_delta_rule(o, r, k, v, w_lin, a_lin, w0, a_bias, state,
+                                  cu_q, state_slot, decay_scale, key_eps)
+            # per-head unit RMS, plain weight, sigmoid output gate
+            _ext().seq_group_rmsnorm(out, o, norm_w, H, eps, g)
+        return out
+    return R.delta_rule(r, k, v, w_lin, a_lin, g, w0, a_bias, norm_w, state,
+                        cu_q, state_slot, decay_scale, key_eps, eps, out_dtype)
+
+
+def ssm_scan(xbc, dt, z, dt_bias, a_log, d_skip, state, cu_q, state_slot,
+             groups: int) -> torch.Tensor:
+    """Selective state-space scan; ``state`` (slots, H, N, P) fp32 in place.
+    step = softplus(dt + dt_bias); S <- exp(-exp(a_log)*step) S + step B x^T;
+    y = S^T C + d_skip*x; returns y * silu(z) as fp32 (N, H*P)."""
+    if xbc.is_cuda:
+        slots, H, Ns, P = state.shape
+        out = torch.empty(xbc.shape[0], H * P, dtype=torch.float32,
+                          device=xbc.device)
+        if xbc.shape[0]:
+            _ext().seq_ssm_scan(out, xbc, dt, z, dt_bias, a_log, d_skip,
+                                state, cu_q, state_slot, groups)
+        return out
+    return R.ssm_scan(xbc, dt, z, dt_bias, a_log, d_skip, state, cu_q,
+                      state_slot, groups)
+
+
+def group_rmsnorm(y, weight, groups: int, eps: float, out_dtype):
+    """RMS-norm each of ``groups`` equal parts of a row by its own root mean
+    square, times weight (D,)."""
+    if y.is_cuda:
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        if y.shape[0]:
+            _ext().seq_group_rmsnorm(out, y, weight, groups, eps,
+                                     torch.Tensor())
+        return out
+    return R.group_rmsnorm(y, weight, groups, eps, out_dtype)
+
+
+def rope_inv_freq(dims: int, base: float, device) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, rounded once to fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (base ** (-2.0 * i / dims)).float().to(device)
+
+
+def rope_partial_(q, offset: int, inv_freq, positions):
+    """Rotate-half RoPE in place on q[..., offset:offset+dims] of a
+    (N, H, Dh) tensor; angle = fp32(position) * inv_freq, fp32 cos/sin."""
+    if q.is_cuda:
+        if q.shape[0] and inv_freq.numel():
+            _ext().seq_rope_partial(q, offset, inv_freq, positions)
+        return q
+    return R.rope_partial_(q, offset, inv_freq, positions)
+
+
+def latent_kv_store(dkv, rank: int, norm_w, eps: float, positions, inv_freq,
+                    cache, slot_mapping) -> None:
+    """Row n of dkv = [latent (rank) | shared key part]: RMS-norm the latent
+    (times norm_w), rotate the key part, and write both into the paged
+    latent cache (pages, page_size, rank+rot) at slot_mapping[n]."""
+    if dkv.is_cuda:
+        if dkv.shape[0]:
+            _ext().seq_latent_kv_store(dkv, rank, norm_w, eps, positions,
+                                       inv_freq, cache, slot_mapping)
+        return
+    R.latent_kv_store(dkv, rank, norm_w, eps, positions, inv_freq, cache,
+                      slot_mapping)
+
+
+def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
+                            positions, window: int, sink, scale: float,
+                            out_dtype) -> torch.Tensor:
+    """Windowed attention of every row against its sequence's paged latent
+    cache: score_j = (q_lat . c_j + q_rot . kr_j) * scale for
+    0 <= pos - j < window; softmax whose denominator also holds exp(sink_h);
+    returns sum_j p_j c_j, (N, H, rank).  All heads share the cache rows."""
+    if q_lat.is_cuda:
+        out = torch.empty(q_lat.shape, dtype=out_dtype, device=q_lat.device)
+        if q_lat.shape[0]:
+            _ext().seq_latent_attention(out, q_lat, q_rot, cache, page_table,
+                                        seq_of_tok, positions, window, sink,
+                                        scale)
+        return out
+    return R.latent_window_attention(q_lat, q_rot, cache, page_table,
+                                     seq_of_tok, positions, window, sink,
+                                     scale, out_dtype)
+
+
+def silu_mul_any(gate, up):
+    """silu(gate) * up for bf16 or fp32 (row-strided views allowed)."""
+    if gate.is_cuda:
+        out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+        if gate.shape[0]:
+            _ext().seq_act_mul(out, gate, up, 0)
+        return out
+    return R.silu_mul_any(gate, up)
+
+
+def sigmoid_mul(x, gate):
+    """x * sigmoid(gate)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        if x.shape[0]:
+            _ext().seq_act_mul(out, gate, x, 1)
+        return out
+    return R.sigmoid_mul(x, gate)
+
+
+def tanh_act(x):
+    """tanh(x) (contiguous result; x may be a column slice)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        if x.shape[0]:
+            _ext().seq_act_mul(out, x, x, 2)
+        return out
+    return R.tanh_act(x)
+
+
+def gelu_tanh_mul_rows(gate, table, tokens, col0: int):
+    """gelu_tanh(gate) * table[tokens, col0:col0+d] for gate (N, d)."""
+    if gate.is_cuda:
+        out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+        if gate.shape[0]:
+            _ext().seq_gelu_mul_rows(out, gate, table, tokens, col0)
+        return out
+    return R.gelu_tanh_mul_rows(gate, table, tokens, col0)
+
+
+def moe_combine_(res, y_sorted, inv_idx, scale: float) -> None:
+    """res[n] += scale * sum_k y_sorted[inv_idx[n, k]] (fp32 residual)."""
+    if res.is_cuda:
+        if res.shape[0]:
+            _ext().seq_moe_combine(res, y_sorted, inv_idx, scale)
+        return
+    R.moe_combine_(res, y_sorted, inv_idx, scale)

@@ -1,0 +1,203 @@
+"""PyTorch forms of the sequence-mixer ops (ops/seq.py): the CPU execution
+path of the no-GPU test tier and the numerics reference of each HIP kernel in
+csrc/seq_*.hip.  Batches are packed: row n belongs to sequence
+``seq_of_tok[n]``; ``cu_q`` bounds each sequence's rows; recurrent state
+lives in ``state[state_slot[b]]`` and is read and written in place.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+
+def _w(weight: torch.Tensor) -> torch.Tensor:
+    return weight.float().reshape(-1)
+
+
+def add_rmsnorm_f32res(res, y, weight, eps, out_dtype):
+    if y is not None:
+        res.add_(y.float())
+    inv = torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps)
+    return (res * inv * _w(weight)).to(out_dtype)
+
+
+def residual_add_cast(res, y, out_dtype):
+    if y is not None:
+        res.add_(y.float())
+    return res if out_dtype == torch.float32 else res.to(out_dtype)
+
+
+def add_scaled_unit_rms(res, y, weight, eps):
+    yf = y.float()
+    inv = torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
+    res.add_(yf * inv * _w(weight))
+
+
+def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,
+                      add_input, act_silu, out_dtype):
+    taps = w.shape[1]
+    C = w.shape[0]
+    out = torch.empty(x.shape[0], C, dtype=out_dtype, device=x.device)
+    cu = cu_q.tolist()
+    wf = w.float()
+    for b, slot in enumerate(state_slot.tolist()):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        xs = x[q0:q1].float()
+        hist = torch.cat([state[slot], xs], 0)          # (taps-1+L, C)
+        y = torch.zeros_like(xs)
+        for j in range(taps):
+            y += wf[:, j] * hist[j:j + (q1 - q0)]
+        if bias is not None:
+            y += bias.float()
+        if add_input:
+            y += xs
+        if act_silu:
+            y = y * torch.sigmoid(y)
+        out[q0:q1] = y.to(out_dtype)
+        if taps > 1:
+            state[slot] = hist[-(taps - 1):]
+    return out
+
+
+def delta_rule(r, k, v, w_lin, a_lin, g, w0, a_bias, norm_w, state, cu_q,
+               state_slot, decay_scale, key_eps, eps, out_dtype):
+    slots, H, Dk, Dv = state.shape
+    N = r.shape[0]
+    out = torch.empty(N, H * Dv, dtype=torch.float32, device=r.device)
+    rf = r.float().view(N, H, Dk)
+    kf = k.float().view(N, H, Dk)
+    vf = v.float().view(N, H, Dv)
+    dec = torch.exp(-decay_scale * torch.sigmoid(
+        w_lin.float() + w0.float())).view(N, H, Dk)
+    rem = torch.sigmoid(a_lin.float() + a_bias.float()).view(N, H, Dk)
+    unit = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + key_eps)
+    cu = cu_q.tolist()
+    for b, slot in enumerate(state_slot.tolist()):
+        S = state[slot]                                  # (H, Dk, Dv)
+        for n in range(cu[b], cu[b + 1]):
+            proj = torch.einsum("hk,hkv->hv", unit[n], S)
+            S = dec[n].unsqueeze(-1) * S \
+                - (rem[n] * unit[n]).unsqueeze(-1) * proj.unsqueeze(1) \
+                + kf[n].unsqueeze(-1) * vf[n].unsqueeze(1)
+            o = torch.einsum("hk,hkv->hv", rf[n], S)
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+            out[n] = o.reshape(-1)
+        state[slot] = S
+    out = out * norm_w.float() * torch.sigmoid(g.float())
+    return out.to(out_dtype)
+
+
+def ssm_scan(xbc, dt, z, dt_bias, a_log, d_skip, state, cu_q, state_slot,
+             groups):
+    slots, H, Ns, P = state.shape
+    N = xbc.shape[0]
+    inner = H * P
+    xf = xbc[:, :inner].float().view(N, H, P)
+    Bf = xbc[:, inner:inner + groups * Ns].float().view(N, groups, Ns)
+    Cf = xbc[:, inner + groups * Ns:].float().view(N, groups, Ns)
+    per = H // groups
+    Bh = Bf.repeat_interleave(per, dim=1)                # (N, H, Ns)
+    Ch = Cf.repeat_interleave(per, dim=1)
+    step = torch.nn.functional.softplus(dt.float() + dt_bias.float(),
+                                        threshold=1e9)   # (N, H), no clamp
+    decay = torch.exp(-torch.exp(a_log.float()) * step)
+    y = torch.empty(N, H, P, dtype=torch.float32, device=xbc.device)
+    cu = cu_q.tolist()
+    for b, slot in enumerate(state_slot.tolist()):
+        S = state[slot]                                  # (H, Ns, P)
+        for n in range(cu[b], cu[b + 1]):
+            S = decay[n].view(H, 1, 1) * S + step[n].view(H, 1, 1) * \
+                Bh[n].unsqueeze(-1) * xf[n].unsqueeze(1)
+            y[n] = torch.einsum("hn,hnp->hp", Ch[n], S) \
+                + d_skip.float().view(H, 1) * xf[n]
+        state[slot] = S
+    zf = z.float()
+    return y.view(N, inner) * (zf * torch.sigmoid(zf))
+
+
+def group_rmsnorm(y, weight, groups, eps, out_dtype):
+    N, D = y.shape
+    yf = y.float().view(N, groups, D // groups)
+    yf = yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
+    return (yf.view(N, D) * weight.float()).to(out_dtype)
+
+
+def _rotate(x, positions, inv_freq):
+    """x (N, ..., dims) rotate-half over the last axis."""
+    half = inv_freq.numel()
+    ang = positions.float().unsqueeze(-1) * inv_freq.float()   # (N, half)
+    while ang.dim() < x.dim():
+        ang = ang.unsqueeze(1)
+    c, s = torch.cos(ang), torch.sin(ang)
+    a, b = x[..., :half].float(), x[..., half:2 * half].float()
+    return torch.cat([a * c - b * s, b * c + a * s], -1)
+
+
+def rope_partial_(q, offset, inv_freq, positions):
+    dims = 2 * inv_freq.numel()
+    if dims == 0:
+        return q
+    part = q[..., offset:offset + dims]
+    part.copy_(_rotate(part, positions, inv_freq).to(q.dtype))
+    return q
+
+
+def latent_kv_store(dkv, rank, norm_w, eps, positions, inv_freq, cache,
+                    slot_mapping):
+    c = dkv[:, :rank].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = dkv[:, rank:].float().clone()
+    dims = 2 * inv_freq.numel()
+    if dims:
+        kr[:, :dims] = _rotate(kr[:, :dims], positions, inv_freq)
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping.long()] = torch.cat([c, kr], -1).to(cache.dtype)
+
+
+def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
+                            positions, window, sink, scale, out_dtype):
+    N, H, R = q_lat.shape
+    ps = cache.shape[1]
+    flat = cache.view(-1, cache.shape[-1]).float()
+    out = torch.empty(N, H, R, dtype=torch.float32, device=q_lat.device)
+    ptab = page_table.tolist()
+    for n, (b, p) in enumerate(zip(seq_of_tok.tolist(), positions.tolist())):
+        lo = max(0, p - window + 1)
+        rows = torch.tensor([ptab[b][j // ps] * ps + j % ps
+                             for j in range(lo, p + 1)], dtype=torch.long)
+        kv = flat[rows]                                  # (L, R + rd)
+        s = (q_lat[n].float() @ kv[:, :R].t()
+             + q_rot[n].float() @ kv[:, R:].t()) * scale   # (H, L)
+        s = torch.cat([s, sink.float().view(H, 1)], 1)
+        pr = torch.softmax(s, -1)[:, :-1]
+        out[n] = pr @ kv[:, :R]
+    return out.to(out_dtype)
+
+
+def silu_mul_any(gate, up):
+    gf = gate.float()
+    return (gf * torch.sigmoid(gf) * up.float()).to(gate.dtype)
+
+
+def sigmoid_mul(x, gate):
+    return (x.float() * torch.sigmoid(gate.float())).to(x.dtype)
+
+
+def tanh_act(x):
+    return torch.tanh(x.float()).to(x.dtype)
+
+
+def gelu_tanh_mul_rows(gate, table, tokens, col0):
+    zf = gate.float()
+    c = math.sqrt(2.0 / math.pi)
+    act = 0.5 * zf * (1.0 + torch.tanh(c * (zf + 0.044715 * zf ** 3)))
+    e = table[tokens.long(), col0:col0 + gate.shape[1]].float()
+    return (act * e).to(gate.dtype)
+
+
+def moe_combine_(res, y_sorted, inv_idx, scale):
+    res.add_(y_sorted.float()[inv_idx.long()].sum(1) * scale)

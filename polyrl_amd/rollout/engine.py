@@ -22,7 +22,8 @@ import torch
 
 import polyrl_amd.ops as ops
 from ..models.registry import DecoderConfig
-from .kv_cache import PagedKVCache, RadixCache
+from .kv_cache import (PagedKVCache, PagedLatentCache, RadixCache,
+                       StateSlots)
 
 
 def _mm_nt(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -369,16 +370,32 @@ class Engine:
                  decode_chunk_size: int = 16,
                  tp_ctx=None,
                  seed: int = 0,
-                 enable_radix_cache: bool = False):
+                 enable_radix_cache: bool = False,
+                 kv_token_capacity: Optional[int] = None):
         self.cfg = cfg
         self.device = device
         self.dtype = dtype
-        self.model = InferenceModel(cfg, device, dtype, tp_ctx=tp_ctx)
+        # hybrid decoders (recurrent / state-space / latent-attention
+        # layers): paged latent rows + per-sequence state slots, and one
+        # mixed batch per step instead of a prefill and a decode pass
+        self.hybrid = bool(getattr(cfg, "is_hybrid", False))
+        if self.hybrid:
+            from .hybrid_model import HybridInferenceModel
+            self.model = HybridInferenceModel(cfg, device, dtype,
+                                              tp_ctx=tp_ctx)
+        else:
+            self.model = InferenceModel(cfg, device, dtype, tp_ctx=tp_ctx)
         self.model._engine_owner = self   # weight publishers flush the radix
         self.tp = self.model.tp
         self.max_running = max_running_requests
         self.max_batched_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len or cfg.max_position_embeddings
+        self.states: Optional[StateSlots] = None
+        self._forced: Dict[str, Request] = {}
+        if self.hybrid:
+            self._init_hybrid(page_size, kv_bytes_budget, kv_token_capacity,
+                              seed, decode_chunk_size)
+            return
         # KV cache holds this rank's local KV heads (gpt2 has no GQA/TP)
         hk_local = (cfg.num_attention_heads if cfg.arch == "gpt2"
                     else cfg.num_key_value_heads // self.tp.size)
@@ -387,6 +404,8 @@ class Engine:
         if kv_bytes_budget is None:
             kv_bytes_budget = 1 << 30  # 1 GiB default (tests); callers size it
         num_pages = max(int(kv_bytes_budget // (bt * page_size)), 8)
+        if kv_token_capacity is not None:
+            num_pages = -(-kv_token_capacity // page_size)
         self.kv = PagedKVCache(cfg.num_hidden_layers, hk_local,
                                cfg.head_dim, num_pages, page_size,
                                dtype=dtype, device=device)
@@ -419,6 +438,40 @@ class Engine:
         # reserved scratch slot and their outputs are discarded.
         self._decode_buckets = bool(int(__import__("os").environ.get(
             "POLYRL_DECODE_BUCKETS", "0")))
+
+    def _init_hybrid(self, page_size, kv_bytes_budget, kv_token_capacity,
+                     seed, decode_chunk_size):
+        """Cache, state pool and scheduler settings of a hybrid decoder:
+        latent rows are paged like KV; every running request also holds one
+        state slot (recurrent states + convolution histories), so the slot
+        pool is as large as the running set."""
+        dev = self.device
+        row_dims = self.model.cache_row_dims()
+        elt = torch.empty(0, dtype=self.dtype).element_size()
+        if kv_token_capacity is not None:
+            num_pages = -(-kv_token_capacity // page_size)
+        else:
+            bt = PagedLatentCache.bytes_per_token_rows(row_dims, elt)
+            budget = (1 << 30) if kv_bytes_budget is None else kv_bytes_budget
+            num_pages = max(int(budget // (bt * page_size)), 8)
+        self.kv = PagedLatentCache(row_dims, num_pages, page_size,
+                                   dtype=self.dtype, device=dev)
+        self.states = StateSlots(self.model.state_shapes(), self.max_running,
+                                 device=dev)
+        self._seq_counter = 0
+        self._seq_ids = {}
+        self.waiting, self.running = [], []
+        self._step_counter = 0
+        self._seed = seed
+        self._abort_all = False
+        self._gen = torch.Generator().manual_seed(seed)
+        self.decode_chunk_size = 1        # one token per mixed step
+        # recurrent state cannot be shared page-wise: no prefix reuse
+        self.enable_prefix_sharing = False
+        self.radix = None
+        self.enable_hip_graphs = False
+        self._graphs, self._graph_pool = {}, None
+        self._decode_buckets = False
 
     # ------------------------------------------------------------ public API
     def add_request(self, rid: str, input_ids: List[int],
@@ -534,7 +587,8 @@ class Engine:
                 radix_pages, radix_len = self.radix.match(nxt.input_ids)
             need = min(len(nxt.input_ids) - nxt.prefill_pos - radix_len,
                        admit_budget)
-            if not self._ensure_pages(need):
+            if not self._ensure_pages(need) or \
+                    (self.states is not None and not self.states.free_slots):
                 if radix_pages:
                     self.kv.unref_pages(radix_pages)
                 break
@@ -543,6 +597,8 @@ class Engine:
             sid = self._seq_counter
             self._seq_counter += 1
             self._seq_ids[nxt.rid] = sid
+            if self.states is not None:
+                self.states.acquire(sid)
             if radix_len:
                 # cached prompt pages seed the page table; prefill resumes
                 # at the page-aligned boundary (chunked-prefill path
@@ -564,12 +620,26 @@ class Engine:
             prefill_reqs.append(r)
             prefill_lens.append(take)
             token_budget -= take
-        if prefill_reqs:
-            self._run_prefill(prefill_reqs, prefill_lens)
-
         # ---- decode ---------------------------------------------------------
         decode_reqs = [r for r in self.running
                        if r.prefill_pos >= len(r.input_ids) and not r.finished]
+        if self.hybrid:
+            ok = []
+            for r in decode_reqs:
+                if self._ensure_pages(1) and \
+                        self.kv.allocate(self._seq_ids[r.rid], 1):
+                    ok.append(r)
+                else:
+                    r.finished = True
+                    r.finish_reason = "abort"
+            if prefill_reqs or ok:
+                self._run_mixed(prefill_reqs, prefill_lens, ok)
+            decode_reqs = []
+        elif prefill_reqs:
+            self._run_prefill(prefill_reqs, prefill_lens)
+            decode_reqs = [r for r in self.running
+                           if r.prefill_pos >= len(r.input_ids)
+                           and not r.finished]
         if decode_reqs:
             ok = []
             for r in decode_reqs:
@@ -636,6 +706,8 @@ class Engine:
                 toks = (r.input_ids + r.output_ids)[:written]
                 self.radix.insert(toks, self.kv._seq_pages.get(sid, []))
             self.kv.free_seq(sid)
+            if self.states is not None:
+                self.states.release(sid)
         if not r.finish_reason:
             r.finish_reason = "length"
         return RequestOutput(rid=r.rid, output_ids=list(r.output_ids),
@@ -686,14 +758,117 @@ class Engine:
                 r.finished = True
                 r.finish_reason = "length"
 
-    def _run_prefill(self, reqs: List[Request], lens: List[int]):
+    # ----------------------------------------------------- hybrid decoders
+    def _hybrid_batch(self, items):
+        """Pack [(request, start, tokens)] into one HybridBatch: pages for
+        the new tokens are already allocated by the caller."""
+        import numpy as np
+        from .hybrid_model import HybridBatch
+        dev = self.device
+        tok, pos, sot, cu, slots, sids, maps = [], [], [], [0], [], [], []
+        for b, (r, start, toks) in enumerate(items):
+            sid = self._seq_ids[r.rid]
+            n = len(toks)
+            tok.extend(toks)
+            pos.extend(range(start, start + n))
+            sot.extend([b] * n)
+            cu.append(cu[-1] + n)
+            slots.append(self.states.slot(sid))
+            sids.append(sid)
+            maps.append(self.kv.slots_for(sid, start, n))
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+        th = np.asarray(tok, dtype=np.int64)
+        return HybridBatch(
+            tokens=torch.from_numpy(th).to(dev), tokens_host=th,
+            positions=i32(pos), seq_of_tok=i32(sot), cu_q=i32(cu),
+            state_slot=i32(slots),
+            slot_mapping=torch.cat(maps).to(dev),
+            page_table=self.kv.page_table(sids).to(dev)), cu
+
+    def _run_mixed(self, prefill_reqs, prefill_lens, decode_reqs):
+        """One forward over prompt portions and single decode tokens
+        together; samples where a prompt completes or a token was decoded."""
+        items = []
+        for r, take in zip(prefill_reqs, prefill_lens):
+            s = r.prefill_pos
+            items.append((r, s, r.input_ids[s:s + take]))
+        for r in decode_reqs:
+            items.append((r, r.seq_len - 1, [r.output_ids[-1]]))
+        bt, cu = self._hybrid_batch(items)
+        res = self.model.forward_batch(bt, self.kv, self.states)
+        rows, reqs = [], []
+        for i, (r, take) in enumerate(zip(prefill_reqs, prefill_lens)):
+            r.prefill_pos += take
+            if r.prefill_pos >= len(r.input_ids):
+                rows.append(cu[i + 1] - 1)
+                reqs.append(r)
+        for j, r in enumerate(decode_reqs):
+            rows.append(cu[len(prefill_reqs) + j + 1] - 1)
+            reqs.append(r)
+        if reqs:
+            idx = torch.tensor(rows, dtype=torch.long, device=self.device)
+            self._sample_last(reqs, res.index_select(0, idx))
+
+    @torch.no_grad()
+    def step_forced(self, entries, end=()):
+        """Teacher-forced step for replaying a trace: ``entries`` is a list
+        of (rid, tokens, want) giving each request's NEXT tokens (a request
+        is admitted at its first entry) and the places among them whose
+        logits are wanted.  All entries run as one batch through the same
+        forward, cache and state pool as :meth:`step`; nothing is sampled.
+        Requests named in ``end`` give back their pages and state slot.
+        Returns fp32 logits (sum of wants, vocab) in entry order."""
+        items, rows, base = [], [], 0
+        for rid, toks, want in entries:
+            r = self._forced.get(rid)
+            if r is None:
+                if self.states is not None and not self.states.free_slots:
+                    raise RuntimeError("no free state slot for " + rid)
+                r = Request(rid=rid, input_ids=[], sampling=SamplingParams())
+                sid = self._seq_counter
+                self._seq_counter += 1
+                self._seq_ids[rid] = sid
+                if self.states is not None:
+                    self.states.acquire(sid)
+                self._forced[rid] = r
+            start = len(r.input_ids)
+            if not self._ensure_pages(len(toks)) or \
+                    not self.kv.allocate(self._seq_ids[rid], len(toks)):
+                raise RuntimeError("cache pool exhausted at " + rid)
+            r.input_ids.extend(toks)
+            r.prefill_pos = len(r.input_ids)
+            items.append((r, start, list(toks)))
+            rows.extend(base + w for w in want)
+            base += len(toks)
+        logits = None
+        if items:
+            if self.hybrid:
+                bt, _ = self._hybrid_batch(items)
+                hidden = self.model.forward_batch(bt, self.kv, self.states)
+            else:
+                hidden = self._forward_portions(
+                    [it[0] for it in items], [it[1] for it in items],
+                    [len(it[2]) for it in items])[0]
+            if rows:
+                idx = torch.tensor(rows, dtype=torch.long, device=self.device)
+                logits = self.model.logits(hidden.index_select(0, idx)).float()
+        for rid in end:
+            r = self._forced.pop(rid, None)
+            if r is not None:
+                r.finish_reason = "stop"
+                self._emit(r)
+        return logits
+
+    def _forward_portions(self, reqs: List[Request], starts: List[int],
+                          lens: List[int]):
+        """Hidden rows of each request's tokens [start, start+len) against
+        its cached history (dense decoders); returns (hidden, cu_q)."""
         dev = self.device
         tok_list, pos_list, slot_list = [], [], []
         cu_q = [0]
         cu_k = [0]
-        for r, take in zip(reqs, lens):
+        for r, start, take in zip(reqs, starts, lens):
             sid = self._seq_ids[r.rid]
-            start = r.prefill_pos
             tok_list.extend(r.input_ids[start:start + take])
             pos_list.extend(range(start, start + take))
             slot_list.append(self.kv.slots_for(sid, start, take))
@@ -704,18 +879,16 @@ class Engine:
         slots = torch.cat(slot_list).to(dev)
         cu_q_t = torch.tensor(cu_q, dtype=torch.int32, device=dev)
         cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
-
         seq_ids = [self._seq_ids[r.rid] for r in reqs]
-        page_table = self.kv.page_table(seq_ids).to(dev)
-        ctx_lens = torch.tensor([s + t for s, t in
-                                 zip((r.prefill_pos for r in reqs), lens)],
+        ctx_lens = torch.tensor([s + t for s, t in zip(starts, lens)],
                                 dtype=torch.int32, device=dev)
+        fresh = all(s == 0 for s in starts)
 
         def attn_fn(li, q, k, v):
-            # chunked prefill: queries attend to the FULL cached history
-            # (cu_k spans include prior chunks) — gather K/V from the cache
-            # pages for this layer.
-            if all(r.prefill_pos == 0 for r in reqs):
+            # portions after the first attend to the FULL cached history
+            # (cu_k spans include earlier portions): gather K/V from the
+            # cache pages of this layer
+            if fresh:
                 return ops.varlen_prefill_attention(q, k, v, cu_q_t, cu_k_t,
                                                     self._scale, causal=True)
             kf, vf = self._gather_kv(li, seq_ids, ctx_lens)
@@ -724,6 +897,12 @@ class Engine:
 
         hidden = self.model.forward_tokens(tokens, positions, self.kv, slots,
                                            attn_fn)
+        return hidden, cu_q
+
+    def _run_prefill(self, reqs: List[Request], lens: List[int]):
+        dev = self.device
+        hidden, cu_q = self._forward_portions(
+            reqs, [r.prefill_pos for r in reqs], lens)
         # requests whose prefill completes sample their first token;
         # group parents fork their children first (shared prompt pages)
         done_rows, done_reqs = [], []

@@ -1,0 +1,502 @@
+"""Engine-side model for hybrid decoders (models/hybrid.py): per-layer weight
+buffers and the no-autograd forward over a packed mixed batch (portions of
+prompts beside single decode tokens) on the sequence-mixer kernels
+(ops/seq.py).
+
+The model owns no cache, no state and no loop over steps: the engine's
+PagedLatentCache / StateSlots hold them and the engine's scheduler builds
+the batch.  Each mixer and feed-forward kind is a small class with its own
+buffers, checkpoint names and state shapes, picked per layer from the
+config, so a further design composes them differently.
+
+Precision: the residual stream, all norms, recurrent states and what enters
+the recurrences stay fp32; projections run in the engine dtype (bf16 or
+fp32) with fp32 accumulation.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+import polyrl_amd.ops as ops
+from polyrl_amd.ops import seq
+from ..models.hybrid import HybridConfig
+
+
+@dataclass
+class HybridBatch:
+    """A packed step: rows [cu_q[b], cu_q[b+1]) are sequence b's next
+    tokens at positions start[b]...; device tensors are int32 unless said."""
+    tokens: torch.Tensor          # (N,) int64
+    tokens_host: np.ndarray       # (N,) int64
+    positions: torch.Tensor       # (N,)
+    seq_of_tok: torch.Tensor      # (N,)
+    cu_q: torch.Tensor            # (B+1,)
+    state_slot: torch.Tensor      # (B,)
+    slot_mapping: torch.Tensor    # (N,) cache row of each token
+    page_table: torch.Tensor      # (B, max_pages)
+
+
+_TUNED = False
+
+
+def set_tuned_products(on: bool) -> None:
+    """Route the next forward's projections through the per-shape pinned
+    hipBLASLt path (worth its one-off search only for the few, recurring
+    shapes of pure decode steps)."""
+    global _TUNED
+    _TUNED = bool(on)
+
+
+def _mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """y = x @ w.T (vendor matrix product, fp32 accumulation)."""
+    if _TUNED and x.is_cuda and x.dtype == torch.bfloat16 \
+            and x.shape[0] <= 512 and x.is_contiguous():
+        return ops.tuned_mm_nt(x, w)
+    return x @ w.t()
+
+
+class _Part:
+    """Buffers of one mixer / feed-forward with their checkpoint names."""
+
+    def named(self, prefix: str) -> Dict[str, torch.Tensor]:
+        raise NotImplementedError
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {}
+
+
+class DeltaRuleMixer(_Part):
+    def __init__(self, spec, width, device, dtype):
+        self.spec = spec
+        self.n = n = spec.heads * spec.dim
+        self.rank = spec.decay_rank
+        z = lambda *s, dt=dtype: torch.empty(*s, device=device, dtype=dt)
+        f32 = torch.float32
+        # one projection for r, k, v, removal rate, output gate, decay-in
+        self.w_in = z(5 * n + self.rank, width)
+        self.w2 = z(n, self.rank)
+        self.w0, self.a_b, self.norm = z(n, dt=f32), z(n, dt=f32), z(n, dt=f32)
+        self.wo = z(width, n)
+
+    def named(self, p):
+        n = self.n
+        return {p + "r": self.w_in[:n], p + "k": self.w_in[n:2 * n],
+                p + "v": self.w_in[2 * n:3 * n], p + "a": self.w_in[3 * n:4 * n],
+                p + "g": self.w_in[4 * n:5 * n], p + "w1": self.w_in[5 * n:],
+                p + "w2": self.w2, p + "w0": self.w0, p + "a.b": self.a_b,
+                p + "norm": self.norm, p + "o": self.wo}
+
+    def state_shapes(self):
+        s = self.spec
+        return {"S": (s.heads, s.dim, s.dim)}
+
+    def forward(self, h, bt, li, model, cache, states):
+        n, s = self.n, self.spec
+        proj = _mm(h, self.w_in)
+        col = lambda i: proj.narrow(1, i * n, n)
+        w_lin = _mm(seq.tanh_act(proj.narrow(1, 5 * n, self.rank)), self.w2)
+        y = seq.delta_rule(col(0), col(1), col(2), w_lin, col(3), col(4),
+                           self.w0, self.a_b, self.norm,
+                           states.tensors[(li, "S")], bt.cu_q, bt.state_slot,
+                           s.decay_scale, s.key_eps, model.cfg.norm_eps,
+                           h.dtype)
+        return _mm(y, self.wo)
+
+
+class SSMMixer(_Part):
+    def __init__(self, spec, width, device, dtype):
+        self.spec = spec
+        z = lambda *s, dt=dtype: torch.empty(*s, device=device, dtype=dt)
+        f32 = torch.float32
+        inner, ch = spec.inner, spec.conv_channels
+        self.w_in = z(inner + ch + spec.heads, width)
+        self.conv = z(ch, spec.conv, dt=f32)
+        self.conv_b = z(ch, dt=f32)
+        self.dt_bias, self.a_log, self.d = (z(spec.heads, dt=f32),
+                                            z(spec.heads, dt=f32),
+                                            z(spec.heads, dt=f32))
+        self.norm = z(inner, dt=f32)
+        self.wo = z(width, inner)
+
+    def named(self, p):
+        return {p + "in": self.w_in, p + "conv": self.conv,
+                p + "conv.b": self.conv_b, p + "dt_bias": self.dt_bias,
+                p + "A_log": self.a_log, p + "D": self.d,
+                p + "norm": self.norm, p + "o": self.wo}
+
+    def state_shapes(self):
+        s = self.spec
+        out = {"S": (s.heads, s.state, s.vdim)}
+        if s.conv > 1:
+            out["conv"] = (s.conv - 1, s.conv_channels)
+        return out
+
+    def forward(self, h, bt, li, model, cache, states):
+        s = self.spec
+        inner, ch = s.inner, s.conv_channels
+        proj = _mm(h, self.w_in)
+        conv_state = model._state(states, (li, "conv"), ch)
+        xbc = seq.causal_conv_state(proj.narrow(1, inner, ch), self.conv,
+                                    self.conv_b, conv_state, bt.cu_q,
+                                    bt.state_slot, bt.seq_of_tok, False, True,
+                                    h.dtype)
+        y = seq.ssm_scan(xbc, proj.narrow(1, inner + ch, s.heads),
+                         proj.narrow(1, 0, inner), self.dt_bias, self.a_log,
+                         self.d, states.tensors[(li, "S")], bt.cu_q,
+                         bt.state_slot, s.groups)
+        y = seq.group_rmsnorm(y, self.norm, s.norm_groups, model.cfg.norm_eps,
+                              h.dtype)
+        return _mm(y, self.wo)
+
+
+class LatentAttnMixer(_Part):
+    def __init__(self, spec, width, device, dtype):
+        self.spec = s = spec
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        f32 = torch.float32
+        self.nq = s.heads * (s.dim + s.rot_dim)
+        self.nv = s.heads * s.vdim
+        self.owner = s.kv_from is None
+        self.row = s.kv_rank + s.rot_dim
+        # one projection for queries, output gate and (if owned) the latent
+        self.w_in = z(self.nq + self.nv + (self.row if self.owner else 0),
+                      width)
+        self.dkv_norm = z(s.kv_rank, dt=f32) if self.owner else None
+        self.uk = z(s.heads * s.dim, s.kv_rank)
+        self.uv = z(s.heads * s.vdim, s.kv_rank)
+        self.sink = z(s.heads, dt=f32)
+        self.wo = z(width, self.nv)
+        self.inv_freq = seq.rope_inv_freq(s.rope_dims, s.rope_base, device)
+
+    def named(self, p):
+        out = {p + "q": self.w_in[:self.nq],
+               p + "g": self.w_in[self.nq:self.nq + self.nv],
+               p + "uk": self.uk, p + "uv": self.uv, p + "sink": self.sink,
+               p + "o": self.wo}
+        if self.owner:
+            out[p + "dkv"] = self.w_in[self.nq + self.nv:]
+            out[p + "dkv.norm"] = self.dkv_norm
+        return out
+
+    def forward(self, h, bt, li, model, cache, states):
+        s = self.spec
+        N, H = h.shape[0], s.heads
+        proj = _mm(h, self.w_in)
+        rows = cache.rows[li if self.owner else s.kv_from]
+        if self.owner:
+            seq.latent_kv_store(proj.narrow(1, self.nq + self.nv, self.row),
+                                s.kv_rank, self.dkv_norm, model.cfg.norm_eps,
+                                bt.positions, self.inv_freq, rows,
+                                bt.slot_mapping)
+        q = proj.narrow(1, 0, self.nq).unflatten(1, (H, s.dim + s.rot_dim))
+        seq.rope_partial_(q, s.dim, self.inv_freq, bt.positions)
+        # absorb the key up-projection into the query: (q . W_uk c) =
+        # (W_uk^T q) . c, so every head scores against the cached latent
+        q_lat = torch.bmm(q[:, :, :s.dim].transpose(0, 1),
+                          self.uk.view(H, s.dim, s.kv_rank)).transpose(0, 1)
+        o_lat = seq.latent_window_attention(
+            q_lat.contiguous(), q[:, :, s.dim:], rows, bt.page_table,
+            bt.seq_of_tok, bt.positions, s.window, self.sink, s.scale,
+            h.dtype)
+        # ... and the value up-projection after the weighted sum
+        o = torch.bmm(o_lat.transpose(0, 1),
+                      self.uv.view(H, s.vdim, s.kv_rank).transpose(1, 2))
+        o = o.transpose(0, 1).reshape(N, self.nv)
+        o = seq.sigmoid_mul(o, proj.narrow(1, self.nq, self.nv))
+        return _mm(o, self.wo)
+
+
+class DenseFF(_Part):
+    def __init__(self, spec, width, vocab, device, dtype):
+        self.ff = spec.ff
+        self.w_gu = torch.empty(2 * spec.ff, width, device=device, dtype=dtype)
+        self.w_down = torch.empty(width, spec.ff, device=device, dtype=dtype)
+
+    def named(self, p):
+        return {p + "gate": self.w_gu[:self.ff], p + "up": self.w_gu[self.ff:],
+                p + "down": self.w_down}
+
+    def forward(self, h, res, bt):
+        gu = _mm(h, self.w_gu)
+        act = seq.silu_mul_any(gu.narrow(1, 0, self.ff),
+                               gu.narrow(1, self.ff, self.ff))
+        return _mm(act, self.w_down)      # added by the caller's next norm
+
+
+class TableMoE(_Part):
+    """Experts chosen by a table over token ids (no router network): the
+    host knows every token's experts before the step runs, so rows are
+    sorted by expert there and the device runs one dense product per
+    expert that has rows."""
+
+    def __init__(self, spec, width, vocab, device, dtype):
+        self.ff, self.E, self.top = spec.ff, spec.experts, spec.top
+        self.w_gu = torch.empty(spec.experts, 2 * spec.ff, width,
+                                device=device, dtype=dtype)
+        self.w_down = torch.empty(spec.experts, width, spec.ff,
+                                  device=device, dtype=dtype)
+        self.table = torch.zeros(vocab, spec.top, device=device,
+                                 dtype=torch.int32)
+        self._table_host: Optional[np.ndarray] = None
+
+    def named(self, p):
+        out = {p + "table": self.table}
+        for e in range(self.E):
+            out[f"{p}e{e}.gate"] = self.w_gu[e, :self.ff]
+            out[f"{p}e{e}.up"] = self.w_gu[e, self.ff:]
+            out[f"{p}e{e}.down"] = self.w_down[e]
+        return out
+
+    def route(self, tokens_host: np.ndarray):
+        if self._table_host is None:
+            self._table_host = self.table.cpu().numpy()
+        flat = self._table_host[tokens_host].reshape(-1)
+        order = np.argsort(flat, kind="stable")
+        counts = np.bincount(flat, minlength=self.E)
+        inv = np.empty(order.size, dtype=np.int32)
+        inv[order] = np.arange(order.size, dtype=np.int32)
+        return (order // self.top).astype(np.int64), counts, \
+            inv.reshape(-1, self.top)
+
+    def forward(self, h, res, bt):
+        src, counts, inv = self.route(bt.tokens_host)
+        dev = h.device
+        xs = h.index_select(0, torch.from_numpy(src).to(dev))
+        ys = torch.empty(xs.shape[0], h.shape[1], device=dev, dtype=h.dtype)
+        o = 0
+        for e in np.nonzero(counts)[0].tolist():
+            c = int(counts[e])
+            gu = _mm(xs[o:o + c], self.w_gu[e])
+            act = seq.silu_mul_any(gu.narrow(1, 0, self.ff),
+                                   gu.narrow(1, self.ff, self.ff))
+            ys[o:o + c] = _mm(act, self.w_down[e])
+            o += c
+        seq.moe_combine_(res, ys, torch.from_numpy(inv).to(dev),
+                         1.0 / self.top)
+        return None                       # already in the residual
+
+
+_MIXERS = {"general_delta": DeltaRuleMixer, "mamba2": SSMMixer,
+           "latent_attention": LatentAttnMixer}
+_FFS = {"dense": DenseFF, "moe": TableMoE}
+
+
+class HybridLayer:
+    def __init__(self, cfg: HybridConfig, li: int, device, dtype):
+        L = cfg.layers[li]
+        W = cfg.hidden_size
+        f32 = torch.float32
+        self.norm1 = torch.empty(1, device=device, dtype=f32)
+        self.norm2 = torch.empty(1, device=device, dtype=f32)
+        self.canon = torch.empty(W, cfg.canon_taps, device=device, dtype=f32)
+        self.mixer = _MIXERS[L.mixer.kind](L.mixer, W, device, dtype)
+        self.ff = None if L.ff is None else \
+            _FFS[L.ff.kind](L.ff, W, cfg.vocab_size, device, dtype)
+        d = cfg.token_side_dim
+        self.side_gate = torch.empty(d, W, device=device, dtype=dtype)
+        self.side_proj = torch.empty(W, d, device=device, dtype=dtype)
+        self.side_norm = torch.empty(W, device=device, dtype=f32)
+
+    def named(self, p: str) -> Dict[str, torch.Tensor]:
+        out = {p + "norm1": self.norm1, p + "canon1": self.canon,
+               p + "side.gate": self.side_gate,
+               p + "side.proj": self.side_proj,
+               p + "side.norm": self.side_norm}
+        out.update(self.mixer.named(p + "mix."))
+        if self.ff is not None:
+            out[p + "norm2"] = self.norm2
+            out.update(self.ff.named(p + "mlp."))
+        return out
+
+
+class HybridInferenceModel:
+    """Weights + packed forward of a hybrid decoder for the rollout engine
+    (same weight-update surface as InferenceModel: ``_name_map``,
+    ``load_state_dict``, ``update_named``)."""
+
+    def __init__(self, cfg: HybridConfig, device="cuda",
+                 dtype=torch.bfloat16, tp_ctx=None):
+        from ..parallel.tp import TPContext
+        self.tp = tp_ctx if tp_ctx is not None else TPContext(None)
+        assert self.tp.size == 1, \
+            "hybrid decoders run one replica per GPU (tp=1)"
+        self.cfg = cfg
+        self.device = device
+        self.dtype = dtype
+        for L in cfg.layers:                 # sizes the config leaves open
+            if L.mixer.kind == "general_delta" and L.mixer.decay_rank is None:
+                L.mixer.decay_rank = max(8, cfg.hidden_size // 12 // 8 * 8)
+        self.layers = [HybridLayer(cfg, li, device, dtype)
+                       for li in range(cfg.num_hidden_layers)]
+        W = cfg.hidden_size
+        self.embed = torch.empty(cfg.vocab_size, W, device=device, dtype=dtype)
+        self.side_embed = torch.empty(
+            cfg.vocab_size, cfg.num_hidden_layers * cfg.token_side_dim,
+            device=device, dtype=dtype)
+        self.final_norm = torch.empty(1, device=device, dtype=torch.float32)
+        self.lm_head = torch.empty(cfg.vocab_size, W, device=device,
+                                   dtype=dtype)
+        self._name_map: Dict[str, torch.Tensor] = {
+            "embed": self.embed, "side.embed": self.side_embed,
+            "final.norm": self.final_norm, "head": self.lm_head}
+        for li, lw in enumerate(self.layers):
+            self._name_map.update(lw.named(f"l{li}."))
+        self.capture_layers: Optional[List[torch.Tensor]] = None
+
+    # ---------------------------------------------------------- geometry
+    @classmethod
+    def resolve_shapes(cls, cfg: HybridConfig, shapes: Dict[str, tuple]):
+        """Fill sizes that only a tensor's shape gives (the rank of the
+        decay projection) from a checkpoint's name -> shape map."""
+        for li, L in enumerate(cfg.layers):
+            if L.mixer.kind == "general_delta":
+                shp = shapes.get(f"l{li}.mix.w1")
+                if shp is not None:
+                    L.mixer.decay_rank = int(shp[0])
+        return cfg
+
+    def cache_row_dims(self) -> Dict[int, int]:
+        return {li: L.mixer.row for li, L in enumerate(self.layers)
+                if isinstance(L.mixer, LatentAttnMixer) and L.mixer.owner}
+
+    def state_shapes(self) -> Dict[tuple, tuple]:
+        out = {}
+        for li, L in enumerate(self.layers):
+            if self.cfg.canon_taps > 1:
+                out[(li, "canon")] = (self.cfg.canon_taps - 1,
+                                      self.cfg.hidden_size)
+            for k, shp in L.mixer.state_shapes().items():
+                out[(li, k)] = shp
+        return out
+
+    # ------------------------------------------------------------ weights
+    def weight_bytes(self) -> int:
+        return sum(v.numel() * v.element_size()
+                   for v in self._name_map.values())
+
+    def _invalidate_host_copies(self):
+        for L in self.layers:
+            if isinstance(L.ff, TableMoE):
+                L.ff._table_host = None
+
+    @torch.no_grad()
+    def load_state_dict(self, sd: Dict[str, torch.Tensor], strict: bool = True):
+        missing = []
+        for name, buf in self._name_map.items():
+            src = sd.get(name)
+            if src is None:
+                missing.append(name)
+                continue
+            if tuple(src.shape) != tuple(buf.shape) and \
+                    src.numel() == buf.numel() and src.dim() == 0:
+                src = src.reshape(buf.shape)
+            if tuple(src.shape) != tuple(buf.shape):
+                raise ValueError(f"{name}: checkpoint shape "
+                                 f"{tuple(src.shape)} != {tuple(buf.shape)}")
+            buf.copy_(src.to(device=buf.device, dtype=buf.dtype))
+        self._invalidate_host_copies()
+        if strict and missing:
+            raise KeyError(f"missing weights: {sorted(missing)[:5]} ...")
+        if strict:
+            extra = set(sd) - set(self._name_map)
+            if extra:
+                raise KeyError(f"unexpected weights: {sorted(extra)[:5]} ...")
+
+    @torch.no_grad()
+    def update_named(self, name: str, tensor: torch.Tensor) -> bool:
+        buf = self._name_map.get(name)
+        if buf is None:
+            return False
+        buf.copy_(tensor.reshape(buf.shape).to(device=buf.device,
+                                               dtype=buf.dtype))
+        self._invalidate_host_copies()
+        return True
+
+    @torch.no_grad()
+    def init_random(self, seed: int = 0):
+        """Random weights of plausible scale (benchmarks, smoke tests)."""
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        for name, buf in self._name_map.items():
+            if buf.dtype == torch.int32:
+                E = self._moe_of(name).E
+                t = torch.stack([torch.randperm(E, generator=g)[:buf.shape[1]]
+                                 for _ in range(buf.shape[0])]).int() \
+                    if buf.shape[0] <= 4096 else \
+                    torch.rand(buf.shape[0], E, generator=g).argsort(1)[
+                        :, :buf.shape[1]].int()
+                buf.copy_(t)
+            elif name.endswith(("norm1", "norm2", "final.norm", ".norm",
+                                "mix.D")):
+                buf.fill_(1.0)
+            elif name.endswith(("A_log", "dt_bias", "w0", "a.b", "sink",
+                                "conv.b")):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.5)
+            elif name.endswith(("canon1", "mix.conv")):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.3)
+            elif name in ("embed", "side.embed"):
+                buf.copy_(torch.randn(buf.shape, generator=g))
+            else:
+                fan = buf.shape[-1]
+                buf.copy_(torch.randn(buf.shape, generator=g) / fan ** 0.5)
+        self._invalidate_host_copies()
+
+    @staticmethod
+    def _state(states, key, channels: int) -> torch.Tensor:
+        """A convolution's history; a one-tap convolution keeps none."""
+        t = states.tensors.get(key)
+        if t is None:
+            t = states.tensors[key] = torch.zeros(
+                states.num_slots, 0, channels, dtype=torch.float32,
+                device=states.device)
+        return t
+
+    def _moe_of(self, name: str) -> "TableMoE":
+        return self.layers[int(name.split(".")[0][1:])].ff
+
+    # ------------------------------------------------------------ forward
+    @torch.no_grad()
+    def forward_batch(self, bt: HybridBatch, cache, states) -> torch.Tensor:
+        """Packed rows through every layer; returns the fp32 residual
+        stream (N, width) before the final norm.  Writes this step's cache
+        rows and advances the sequences' recurrent states in place."""
+        cfg, dt = self.cfg, self.dtype
+        eps = cfg.norm_eps
+        res = self.embed[bt.tokens].float()
+        pending = None                      # mixer/ff output not yet added
+        d = cfg.token_side_dim
+        for li, L in enumerate(self.layers):
+            h = seq.add_rmsnorm_f32res(res, pending, L.norm1, eps, dt)
+            h = seq.causal_conv_state(
+                h, L.canon, None, self._state(states, (li, "canon"),
+                                              cfg.hidden_size),
+                bt.cu_q, bt.state_slot, bt.seq_of_tok, True, False, dt)
+            pending = L.mixer.forward(h, bt, li, self, cache, states)
+            if L.ff is not None:
+                h = seq.add_rmsnorm_f32res(res, pending, L.norm2, eps, dt)
+                pending = L.ff.forward(h, res, bt)
+            x = seq.residual_add_cast(res, pending, dt)
+            pending = None
+            if d > 0:
+                gate = _mm(x, L.side_gate)
+                gated = seq.gelu_tanh_mul_rows(gate, self.side_embed,
+                                               bt.tokens, li * d)
+                seq.add_scaled_unit_rms(res, _mm(gated, L.side_proj),
+                                        L.side_norm, eps)
+            if self.capture_layers is not None:
+                self.capture_layers.append(res.clone())
+        return res
+
+    @torch.no_grad()
+    def logits(self, res_rows: torch.Tensor) -> torch.Tensor:
+        """Final norm + head on residual rows -> fp32 logits."""
+        h = seq.add_rmsnorm_f32res(res_rows.contiguous(), None,
+                                   self.final_norm, self.cfg.norm_eps,
+                                   self.dtype)
+        out = _mm(h, self.lm_head).float()
+        if self.cfg.logit_scale != 1.0:
+            out = out * self.cfg.logit_scale
+        return out

@@ -13,26 +13,15 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 
-class PagedKVCache:
-    def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int,
-                 num_pages: int, page_size: int = 16,
-                 dtype: torch.dtype = torch.bfloat16, device: str = "cuda"):
-        self.num_layers = num_layers
-        self.num_kv_heads = num_kv_heads
-        self.head_dim = head_dim
+class PageAllocator:
+    """Free-list page allocator with per-sequence page lists and refcounts;
+    the tensors that the pages index belong to the subclasses."""
+
+    def __init__(self, num_pages: int, page_size: int = 16,
+                 device: str = "cuda"):
         self.num_pages = num_pages
         self.page_size = page_size
         self.device = device
-        self.k_cache = [
-            torch.zeros(num_pages, page_size, num_kv_heads, head_dim,
-                        dtype=dtype, device=device)
-            for _ in range(num_layers)
-        ]
-        self.v_cache = [
-            torch.zeros(num_pages, page_size, num_kv_heads, head_dim,
-                        dtype=dtype, device=device)
-            for _ in range(num_layers)
-        ]
         self._free: List[int] = list(range(num_pages - 1, -1, -1))
         self._seq_pages: Dict[int, List[int]] = {}
         self._seq_len: Dict[int, int] = {}
@@ -173,6 +162,94 @@ class PagedKVCache:
             pages = self._seq_pages[s]
             pt[i, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
         return pt
+
+
+class PagedKVCache(PageAllocator):
+    """K and V pages per layer, (num_pages, page_size, Hk, D)."""
+
+    def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int,
+                 num_pages: int, page_size: int = 16,
+                 dtype: torch.dtype = torch.bfloat16, device: str = "cuda"):
+        super().__init__(num_pages, page_size, device)
+        self.num_layers = num_layers
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.k_cache = [
+            torch.zeros(num_pages, page_size, num_kv_heads, head_dim,
+                        dtype=dtype, device=device)
+            for _ in range(num_layers)
+        ]
+        self.v_cache = [
+            torch.zeros(num_pages, page_size, num_kv_heads, head_dim,
+                        dtype=dtype, device=device)
+            for _ in range(num_layers)
+        ]
+
+
+class PagedLatentCache(PageAllocator):
+    """One row per token and owning layer: ``rows[li]`` is
+    (num_pages, page_size, row_dim[li]) for every layer li that writes a
+    latent cache (normed latent followed by the rotated shared key part).
+    Layers that read another layer's cache hold no tensor of their own."""
+
+    def __init__(self, row_dims: Dict[int, int], num_pages: int,
+                 page_size: int = 16, dtype: torch.dtype = torch.bfloat16,
+                 device: str = "cuda"):
+        super().__init__(num_pages, page_size, device)
+        self.row_dims = dict(row_dims)
+        self.rows: Dict[int, torch.Tensor] = {
+            li: torch.zeros(num_pages, page_size, d, dtype=dtype,
+                            device=device)
+            for li, d in row_dims.items()}
+
+    @staticmethod
+    def bytes_per_token_rows(row_dims: Dict[int, int],
+                             dtype_bytes: int = 2) -> int:
+        return max(sum(row_dims.values()) * dtype_bytes, 1)
+
+
+class StateSlots:
+    """Fixed pool of per-sequence state slots for recurrent layers and
+    stateful convolutions.  ``tensors[key]`` is (num_slots, *shape) fp32;
+    a slot is zeroed when it is handed out, so a sequence always starts
+    from the zero state whatever the slot held before."""
+
+    def __init__(self, shapes: Dict[object, tuple], num_slots: int,
+                 device: str = "cuda"):
+        self.num_slots = num_slots
+        self.device = device
+        self.tensors: Dict[object, torch.Tensor] = {
+            key: torch.zeros(num_slots, *shape, dtype=torch.float32,
+                             device=device)
+            for key, shape in shapes.items()}
+        self._free: List[int] = list(range(num_slots - 1, -1, -1))
+        self._slot_of: Dict[int, int] = {}
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free)
+
+    def bytes_per_slot(self) -> int:
+        return sum(t[0].numel() * 4 for t in self.tensors.values())
+
+    def acquire(self, seq_id: int) -> Optional[int]:
+        """Slot for a new sequence (zeroed), or None when all are taken."""
+        assert seq_id not in self._slot_of
+        if not self._free:
+            return None
+        slot = self._free.pop()
+        for t in self.tensors.values():
+            t[slot].zero_()
+        self._slot_of[seq_id] = slot
+        return slot
+
+    def slot(self, seq_id: int) -> int:
+        return self._slot_of[seq_id]
+
+    def release(self, seq_id: int) -> None:
+        slot = self._slot_of.pop(seq_id, None)
+        if slot is not None:
+            self._free.append(slot)
 
 
 class _RadixNode:

@@ -1,9 +1,11 @@
-"""In-tree build of the polyrl_amd HIP extension for gfx950 (MI355X).
+"""In-tree build of the polyrl_amd HIP extensions for gfx950 (MI355X).
 
     PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace
 
-The built .so lands next to the package (polyrl_amd/_hip_C*.so) so it travels
-with a repo snapshot to GPU boxes.
+Two modules land next to the package so they travel with a repo snapshot to
+GPU boxes: ``polyrl_amd._hip`` (dense-decoder engine + trainer kernels) and
+``polyrl_amd._hip_seq`` (sequence-mixer kernels of the hybrid decoders).
+``POLYRL_EXT=seq`` (or ``core``) builds only that one.
 """
 import glob
 import os
@@ -21,36 +23,34 @@ from torch.utils.cpp_extension import BuildExtension, CUDAExtension
 
 CSRC = os.path.join("polyrl_amd", "ops", "csrc")
 
-sources = [
-    os.path.join(CSRC, f)
-    for f in (
-        "bindings.cpp",
-        "gemm_tuned.cpp",
-        "elementwise.hip",
-        "rmsnorm_train.hip",
-        "rope_train.hip",
-        "logprobs.hip",
-        "sampling.hip",
-        "kv_cache.hip",
-        "attention_decode.hip",
-        "attention_prefill.hip",
-        "attention_backward.hip",
-        "attention_backward_v3.hip",
-    )
-]
+CORE = ("bindings.cpp", "gemm_tuned.cpp", "elementwise.hip",
+        "rmsnorm_train.hip", "rope_train.hip", "logprobs.hip", "sampling.hip",
+        "kv_cache.hip", "attention_decode.hip", "attention_prefill.hip",
+        "attention_backward.hip", "attention_backward_v3.hip")
+SEQ = ("seq_bindings.cpp", "seq_ops.hip", "seq_scan.hip", "seq_attn.hip")
+
+# scalar fp32 code only: the compiler must not form packed-fp32 VALU ops
+HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def ext(name, files, libraries=()):
+    return CUDAExtension(
+        name=name, sources=[os.path.join(CSRC, f) for f in files],
+        libraries=list(libraries),
+        extra_compile_args={"cxx": ["-O3", "-std=c++17"],
+                            "nvcc": list(HIPCC_FLAGS)})
+
+
+which = os.environ.get("POLYRL_EXT", "all")
+modules = []
+if which in ("all", "core"):
+    modules.append(ext("polyrl_amd._hip", CORE, ["hipblaslt"]))
+if which in ("all", "seq"):
+    modules.append(ext("polyrl_amd._hip_seq", SEQ))
 
 setup(
     name="polyrl_amd_hip",
-    ext_modules=[
-        CUDAExtension(
-            name="polyrl_amd._hip",
-            sources=sources,
-            libraries=["hipblaslt"],
-            extra_compile_args={
-                "cxx": ["-O3", "-std=c++17"],
-                "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"],
-            },
-        )
-    ],
+    ext_modules=modules,
     cmdclass={"build_ext": BuildExtension.with_options(no_python_abi_suffix=False)},
 )
