@@ -1,0 +1,212 @@
+"""HIP sequence-mixer kernels (csrc/seq_*.hip) against their plain PyTorch
+fp32 forms (ops/seq_ref.py) on packed batches of unequal portions, in bf16
+and fp32, with odd sizes that exercise every guard (rows per lane, columns
+per wave, latent-row chunks, partial key blocks)."""
+import math
+
+import pytest
+import torch
+
+from polyrl_amd.ops import seq
+from polyrl_amd.ops import seq_ref as R
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dt):
+    return dict(rtol=2e-2, atol=2e-2) if dt == torch.bfloat16 else \
+        dict(rtol=2e-5, atol=2e-5)
+
+
+def batch(lens, slots):
+    cu = [0]
+    sot = []
+    for b, n in enumerate(lens):
+        cu.append(cu[-1] + n)
+        sot += [b] * n
+    i32 = lambda x, d: torch.tensor(x, dtype=torch.int32, device=d)
+    return {d: (i32(cu, d), i32(slots, d), i32(sot, d)) for d in ("cpu", DEV)}
+
+
+def rnd(*s, dt=torch.float32, scale=1.0, seed=None):
+    return (torch.randn(*s) * scale).to(dt)
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    torch.manual_seed(1234)
+    assert seq.seq_extension_loaded(), "polyrl_amd._hip_seq must be built"
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("D,wn", [(192, 1), (200, 200), (2048, 1)])
+def test_add_rmsnorm_modes(dt, D, wn):
+    N = 7
+    res, y, w = rnd(N, D), rnd(N, D, dt=dt), rnd(wn).abs() + 0.5
+    r0, r1 = res.clone(), res.clone().to(DEV)
+    want = R.add_rmsnorm_f32res(r0, y, w, 1e-6, dt)
+    got = seq.add_rmsnorm_f32res(r1, y.to(DEV), w.to(DEV), 1e-6, dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-6, atol=1e-6)
+    # no-add form leaves the residual alone
+    got2 = seq.add_rmsnorm_f32res(r1, None, w.to(DEV), 1e-6, dt)
+    torch.testing.assert_close(r1.cpu(), r0, rtol=0, atol=0)
+    torch.testing.assert_close(
+        got2.cpu().float(), R.add_rmsnorm_f32res(r0, None, w, 1e-6, dt).float(),
+        **tol(dt))
+    x = seq.residual_add_cast(r1, y.to(DEV), dt)
+    xw = R.residual_add_cast(r0, y, dt)
+    torch.testing.assert_close(x.cpu().float(), xw.float(), **tol(dt))
+    wv = rnd(D).abs() + 0.5
+    seq.add_scaled_unit_rms(r1, y.to(DEV), wv.to(DEV), 1e-6)
+    R.add_scaled_unit_rms(r0, y, wv, 1e-6)
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("taps,lens", [(4, [5, 1, 2, 9]), (1, [3, 1]),
+                                       (6, [2, 2, 1, 7])])
+def test_causal_conv_state_portions(dt, taps, lens):
+    C, slots = 300, [3, 0, 5, 1][:len(lens)]
+    bt = batch(lens, slots)
+    N = sum(lens)
+    big = rnd(N, C + 40, dt=dt)
+    w, bias = rnd(C, taps, scale=0.5), rnd(C)
+    st0 = rnd(6, taps - 1, C)
+    for add, silu, b in [(True, False, None), (False, True, bias)]:
+        sc, sg = st0.clone(), st0.clone().to(DEV)
+        want = R.causal_conv_state(big[:, 17:17 + C], w, b, sc, *bt["cpu"],
+                                   add, silu, dt)
+        got = seq.causal_conv_state(
+            big.to(DEV)[:, 17:17 + C], w.to(DEV),
+            None if b is None else b.to(DEV), sg, *bt[DEV], add, silu, dt)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+        torch.testing.assert_close(sg.cpu(), sc, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,Dk,lens", [(3, 32, [6, 1, 3]), (2, 24, [4, 1]),
+                                       (2, 80, [1, 5]), (1, 128, [3])])
+def test_delta_rule_scan(dt, H, Dk, lens):
+    Dv = Dk
+    slots = [2, 0, 3][:len(lens)]
+    bt = batch(lens, slots)
+    N, n = sum(lens), H * Dk
+    big = rnd(N, 6 * n, dt=dt)
+    col = lambda t, i: t[:, i * n:(i + 1) * n]
+    w0, ab, nw = rnd(n), rnd(n), rnd(n).abs() + 0.5
+    st0 = rnd(4, H, Dk, Dv, scale=0.3)
+    sc, sg = st0.clone(), st0.clone().to(DEV)
+    args = lambda t, d: [col(t, i) for i in range(6)]
+    a = args(big, "cpu")
+    want = R.delta_rule(*a, w0, ab, nw, sc, bt["cpu"][0], bt["cpu"][1],
+                        math.exp(-0.5), 1e-6, 1e-6, dt)
+    g = args(big.to(DEV), DEV)
+    got = seq.delta_rule(*g, w0.to(DEV), ab.to(DEV), nw.to(DEV), sg,
+                         bt[DEV][0], bt[DEV][1], math.exp(-0.5), 1e-6, 1e-6,
+                         dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(sg.cpu(), sc, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,P,Ns,G,lens", [(6, 32, 48, 1, [5, 1, 2]),
+                                           (4, 24, 16, 2, [1, 7]),
+                                           (4, 80, 128, 4, [3])])
+def test_ssm_scan(dt, H, P, Ns, G, lens):
+    slots = [1, 3, 0][:len(lens)]
+    bt = batch(lens, slots)
+    N, inner = sum(lens), H * P
+    ch = inner + 2 * G * Ns
+    big = rnd(N, inner + ch + H, dt=dt)
+    z, xbc, dtt = big[:, :inner], big[:, inner:inner + ch], big[:, inner + ch:]
+    dtb, al, dk = rnd(H), rnd(H, scale=0.5), rnd(H)
+    st0 = rnd(4, H, Ns, P, scale=0.3)
+    sc, sg = st0.clone(), st0.clone().to(DEV)
+    want = R.ssm_scan(xbc, dtt, z, dtb, al, dk, sc, bt["cpu"][0],
+                      bt["cpu"][1], G)
+    bg = big.to(DEV)
+    got = seq.ssm_scan(bg[:, inner:inner + ch], bg[:, inner + ch:],
+                       bg[:, :inner], dtb.to(DEV), al.to(DEV), dk.to(DEV), sg,
+                       bt[DEV][0], bt[DEV][1], G)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(sg.cpu(), sc, rtol=1e-4, atol=1e-4)
+    for groups in (1, H):
+        nw = rnd(inner).abs() + 0.5
+        torch.testing.assert_close(
+            seq.group_rmsnorm(got, nw.to(DEV), groups, 1e-6, dt).cpu().float(),
+            R.group_rmsnorm(want, nw, groups, 1e-6, dt).float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,R_,rd,dims,window", [(3, 64, 16, 16, 5),
+                                                 (2, 40, 24, 16, 40),
+                                                 (2, 200, 32, 32, 7)])
+def test_latent_store_and_attention(dt, H, R_, rd, dims, window):
+    ps, pages = 4, 40
+    lens, starts = [9, 1, 3], [0, 21, 6]       # portions at these offsets
+    # sequences hold start+len tokens; scatter their pages on purpose
+    perm = torch.randperm(pages).tolist()
+    ptab, used = [], 0
+    for s, n in zip(starts, lens):
+        need = -(-(s + n) // ps)
+        ptab.append(perm[used:used + need] + [0] * (10 - need))
+        used += need
+    ptab_t = torch.tensor(ptab, dtype=torch.int32)
+    inv = seq.rope_inv_freq(dims, 10000.0, "cpu")
+    cache = rnd(pages, ps, R_ + rd, dt=dt)     # "history" = random rows
+    pos, sot, slot = [], [], []
+    for b, (s, n) in enumerate(zip(starts, lens)):
+        for p in range(s, s + n):
+            pos.append(p)
+            sot.append(b)
+            slot.append(ptab[b][p // ps] * ps + p % ps)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    N = len(pos)
+    dkv, nw = rnd(N, R_ + rd + 8, dt=dt), rnd(R_).abs() + 0.5
+    cc, cg = cache.clone(), cache.clone().to(DEV)
+    R.latent_kv_store(dkv[:, 8:], R_, nw, 1e-6, i32(pos), inv, cc, i32(slot))
+    seq.latent_kv_store(dkv.to(DEV)[:, 8:], R_, nw.to(DEV), 1e-6,
+                        i32(pos).to(DEV), inv.to(DEV), cg, i32(slot).to(DEV))
+    torch.testing.assert_close(cg.cpu().float(), cc.float(), **tol(dt))
+    q = rnd(N, H, 20 + rd, dt=dt)
+    qc, qg = q.clone(), q.clone().to(DEV)
+    R.rope_partial_(qc, 20, inv, i32(pos))
+    seq.rope_partial_(qg, 20, inv.to(DEV), i32(pos).to(DEV))
+    torch.testing.assert_close(qg.cpu().float(), qc.float(), **tol(dt))
+    q_lat, sink = rnd(N, H, R_, dt=dt, scale=0.3), rnd(H)
+    want = R.latent_window_attention(q_lat, qc[:, :, 20:], cc, ptab_t,
+                                     i32(sot), i32(pos), window, sink, 0.2,
+                                     dt)
+    got = seq.latent_window_attention(
+        q_lat.to(DEV), qc.to(DEV)[:, :, 20:], cc.to(DEV), ptab_t.to(DEV),
+        i32(sot).to(DEV), i32(pos).to(DEV), window, sink.to(DEV), 0.2, dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_activations_and_combine(dt):
+    N, C = 11, 72
+    big = rnd(N, 2 * C + 5, dt=dt)
+    a, b = big[:, 3:3 + C], big[:, 3 + C:3 + 2 * C]
+    ag, bg = big.to(DEV)[:, 3:3 + C], big.to(DEV)[:, 3 + C:3 + 2 * C]
+    for f, rf in [(seq.silu_mul_any, R.silu_mul_any),
+                  (seq.sigmoid_mul, R.sigmoid_mul)]:
+        torch.testing.assert_close(f(ag, bg).cpu().float(),
+                                   rf(a, b).float(), **tol(dt))
+    torch.testing.assert_close(seq.tanh_act(ag).cpu().float(),
+                               R.tanh_act(a).float(), **tol(dt))
+    table, tok = rnd(50, 3 * C, dt=dt), torch.randint(0, 50, (N,))
+    torch.testing.assert_close(
+        seq.gelu_tanh_mul_rows(ag, table.to(DEV), tok.to(DEV), C).cpu().float(),
+        R.gelu_tanh_mul_rows(a, table, tok, C).float(), **tol(dt))
+    top = 3
+    y = rnd(N * top, C, dt=dt)
+    inv = torch.randperm(N * top).view(N, top).int()
+    r0 = rnd(N, C)
+    r1 = r0.clone().to(DEV)
+    R.moe_combine_(r0, y, inv, 1.0 / top)
+    seq.moe_combine_(r1, y.to(DEV), inv.to(DEV), 1.0 / top)
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
