@@ -44,6 +44,76 @@ import torch
 import torch.distributed as dist
 
 
+def _engine_rates(name, prefill, decode, warmup, steps):
+    """Prefill and decode tokens/s of one registry model on the rollout
+    engine (single GPU, random weights, greedy sampling off: T=1)."""
+    from polyrl_amd.models import get_model_config
+    from polyrl_amd.rollout.engine import Engine, SamplingParams
+    device = "cuda" if torch.cuda.is_available() else "cpu"
+    dtype = torch.bfloat16 if device == "cuda" else torch.float32
+    cfg = get_model_config(name)
+    (pn, pl), (dn, dl) = prefill, decode
+    cap = max(pn * (pl + 16), dn * (dl + 32)) + 1024
+    eng = Engine(cfg, device=device, dtype=dtype, page_size=16,
+                 kv_token_capacity=cap, max_running_requests=max(pn, dn),
+                 max_num_batched_tokens=pn * pl)
+    if getattr(cfg, "is_hybrid", False):
+        eng.model.init_random(0)
+    else:
+        for t in eng.model._name_map.values():
+            t.normal_(0, 0.02)
+    g = torch.Generator().manual_seed(0)
+    mk = lambda n, l: [torch.randint(0, cfg.vocab_size, (l,), generator=g)
+                       .tolist() for _ in range(n)]
+    sync = torch.cuda.synchronize if device == "cuda" else (lambda: None)
+
+    def timed(prompts, new):
+        sync()
+        t0 = time.perf_counter()
+        eng.generate(prompts, SamplingParams(temperature=1.0,
+                                             max_new_tokens=new), "b")
+        sync()
+        return time.perf_counter() - t0
+
+    pre, dec = [], []
+    for i in range(warmup + steps):
+        tp = timed(mk(pn, pl), 1)
+        short = mk(dn, 16)
+        t1 = timed(short, 1)
+        t2 = timed(short, dl + 1)
+        if i >= warmup:
+            pre.append(pn * pl / tp)
+            dec.append(dn * dl / max(t2 - t1, 1e-9))
+    params = sum(v.numel() for v in eng.model._name_map.values())
+    return {"model": name, "params": params,
+            "prefill_tok_s": sum(pre) / len(pre),
+            "decode_tok_s": sum(dec) / len(dec),
+            "decode_ms_per_step": 1e3 * dn / (sum(dec) / len(dec))}
+
+
+def engine_compare(args):
+    """--engine-compare: one JSON line per model and one per pair."""
+    shape = lambda s: tuple(int(x) for x in s.lower().split("x"))
+    prefill, decode = shape(args.engine_prefill), shape(args.engine_decode)
+    for pair in args.engine_compare.split(","):
+        names = pair.split(":")
+        rows = [_engine_rates(n, prefill, decode, args.warmup, args.steps)
+                for n in names]
+        for r in rows:
+            print(json.dumps(r), flush=True)
+        if len(rows) == 2:
+            a, b = rows
+            print(json.dumps({
+                "metric": "rollout-engine tokens/s, hybrid beside dense",
+                "pair": names, "prefill": "%dx%d" % prefill,
+                "decode": "%dx%d" % decode,
+                "prefill_ratio": a["prefill_tok_s"] / b["prefill_tok_s"],
+                "decode_ratio": a["decode_tok_s"] / b["decode_tok_s"],
+                "dtype": "bf16" if torch.cuda.is_available() else "fp32",
+                "data": "synthetic prompts, random-init weights"}),
+                flush=True)
+
+
 def main():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -57,7 +127,19 @@ def main():
     p.add_argument("--prompt-len", type=int, default=256)
     p.add_argument("--response-len", type=int, default=256)
     p.add_argument("--adv", type=str, default="gae", choices=["gae", "grpo"])
+    p.add_argument("--engine-compare", type=str, default=None,
+                   metavar="HYBRID:DENSE[,HYBRID:DENSE...]",
+                   help="instead of the PPO step: rollout-engine prefill and "
+                        "decode tokens/s of a hybrid decoder beside a dense "
+                        "one of equal width and depth (registry names, "
+                        "random weights), e.g. bizusun-1b:llama3-1b")
+    p.add_argument("--engine-prefill", type=str, default="8x2048",
+                   help="engine-compare prefill workload: prompts x length")
+    p.add_argument("--engine-decode", type=str, default="64x128",
+                   help="engine-compare decode workload: batch x new tokens")
     args = p.parse_args()
+    if args.engine_compare:
+        return engine_compare(args)
 
     # distributed init (driver launches via torch.distributed.run for N>1)
     world, rank = 1, 0

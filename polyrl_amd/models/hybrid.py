@@ -116,13 +116,14 @@ class HybridConfig:
             m = L.mixer
             if m.kind == "latent_attention" and m.kv_from is not None:
                 src = self.layers[m.kv_from].mixer
-                assert m.kv_from < li and src.kind == "latent_attention" \
-                    and src.kv_from is None, \
-                    f"layer {li}: kv_from must name an earlier owning layer"
-                assert (src.kv_rank, src.rot_dim, src.rope_dims,
-                        src.rope_base) == (m.kv_rank, m.rot_dim, m.rope_dims,
-                                           m.rope_base), \
-                    f"layer {li}: shared cache needs equal latent geometry"
+                if not (0 <= m.kv_from < li) or \
+                        src.kind != "latent_attention" or \
+                        src.kv_from is not None:
+                    raise ValueError(f"layer {li}: kv_from must name an "
+                                     "earlier layer that owns its cache")
+                if (src.kv_rank, src.rot_dim) != (m.kv_rank, m.rot_dim):
+                    raise ValueError(f"layer {li}: a shared cache needs "
+                                     "equal latent and rotated sizes")
             if m.kind == "mamba2":
                 assert m.heads % m.groups == 0
                 assert m.inner % m.norm_groups == 0

@@ -401,10 +401,6 @@ class HybridInferenceModel:
         self._invalidate_host_copies()
         if strict and missing:
             raise KeyError(f"missing weights: {sorted(missing)[:5]} ...")
-        if strict:
-            extra = set(sd) - set(self._name_map)
-            if extra:
-                raise KeyError(f"unexpected weights: {sorted(extra)[:5]} ...")
 
     @torch.no_grad()
     def update_named(self, name: str, tensor: torch.Tensor) -> bool:
