@@ -41,6 +41,9 @@ void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
                           torch::Tensor page_table, torch::Tensor seq_of_tok,
                           torch::Tensor positions, int64_t window,
                           torch::Tensor sink, double scale);
+void seq_moe_table_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
+                       torch::Tensor tokens, torch::Tensor table,
+                       torch::Tensor w_gu, torch::Tensor w_down);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("seq_add_rmsnorm", &seq_add_rmsnorm,
@@ -58,6 +61,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "gelu_tanh(gate) * table rows gathered by token");
   m.def("seq_moe_combine", &seq_moe_combine,
         "residual += scale * sum of a token's expert rows");
+  m.def("seq_moe_table_ffn", &seq_moe_table_ffn,
+        "table-routed expert feed-forward for decode-sized bf16 batches");
   m.def("seq_delta_rule", &seq_delta_rule,
         "generalised delta rule scan (fp32 state, in place)");
   m.def("seq_ssm_scan", &seq_ssm_scan,

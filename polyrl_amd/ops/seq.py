@@ -243,3 +243,24 @@ def moe_combine_(res, y_sorted, inv_idx, scale: float) -> None:
             _ext().seq_moe_combine(res, y_sorted, inv_idx, scale)
         return
     R.moe_combine_(res, y_sorted, inv_idx, scale)
+
+
+def moe_table_ffn_supported(h, top: int, ff: int) -> bool:
+    """The fused expert path serves bf16 decode-sized batches on the GPU."""
+    return (h.is_cuda and h.dtype == torch.bfloat16
+            and h.shape[0] * top <= 1024 and h.shape[1] % 32 == 0
+            and ff % 32 == 0)
+
+
+def moe_table_ffn(h, tokens, table, w_gu, w_down) -> torch.Tensor:
+    """Table-routed gated experts: row t*top+k of the result is expert
+    table[tokens[t], k] applied to h[t] (silu(Wg h) * (Wu h), then Wd).
+    w_gu (E, 2*ff, W) holds gate rows then up rows; w_down (E, W, ff)."""
+    N, top = h.shape[0], table.shape[1]
+    if h.is_cuda:
+        y = torch.empty(N * top, h.shape[1], dtype=h.dtype, device=h.device)
+        act = torch.empty(N * top, w_down.shape[2], dtype=h.dtype,
+                          device=h.device)
+        _ext().seq_moe_table_ffn(y, act, h, tokens, table, w_gu, w_down)
+        return y
+    return R.moe_table_ffn(h, tokens, table, w_gu, w_down)

@@ -201,3 +201,15 @@ def gelu_tanh_mul_rows(gate, table, tokens, col0):
 
 def moe_combine_(res, y_sorted, inv_idx, scale):
     res.add_(y_sorted.float()[inv_idx.long()].sum(1) * scale)
+
+
+def moe_table_ffn(h, tokens, table, w_gu, w_down):
+    N, top = h.shape[0], table.shape[1]
+    ff = w_down.shape[2]
+    y = torch.empty(N * top, h.shape[1], dtype=h.dtype, device=h.device)
+    for t in range(N):
+        for k, e in enumerate(table[tokens[t]].tolist()):
+            gu = w_gu[e].float() @ h[t].float()
+            a = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(h.dtype)
+            y[t * top + k] = (w_down[e].float() @ a.float()).to(h.dtype)
+    return y

@@ -242,6 +242,7 @@ class TableMoE(_Part):
         self.table = torch.zeros(vocab, spec.top, device=device,
                                  dtype=torch.int32)
         self._table_host: Optional[np.ndarray] = None
+        self._slots: Dict[int, torch.Tensor] = {}
 
     def named(self, p):
         out = {p + "table": self.table}
@@ -262,7 +263,24 @@ class TableMoE(_Part):
         return (order // self.top).astype(np.int64), counts, \
             inv.reshape(-1, self.top)
 
+    def _slot_index(self, n: int, device) -> torch.Tensor:
+        t = self._slots.get(n)
+        if t is None:
+            t = self._slots[n] = torch.arange(
+                n * self.top, dtype=torch.int32, device=device
+            ).view(n, self.top)
+        return t
+
     def forward(self, h, res, bt):
+        if h.shape[0] <= 256 and \
+                seq.moe_table_ffn_supported(h, self.top, self.ff):
+            # decode-sized bf16 batch: routing, both products and the
+            # activation run in two launches, weight-read bound
+            y = seq.moe_table_ffn(h, bt.tokens, self.table, self.w_gu,
+                                  self.w_down)
+            seq.moe_combine_(res, y, self._slot_index(h.shape[0], h.device),
+                             1.0 / self.top)
+            return None
         src, counts, inv = self.route(bt.tokens_host)
         dev = h.device
         xs = h.index_select(0, torch.from_numpy(src).to(dev))

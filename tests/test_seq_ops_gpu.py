@@ -210,3 +210,22 @@ def test_activations_and_combine(dt):
     R.moe_combine_(r0, y, inv, 1.0 / top)
     seq.moe_combine_(r1, y.to(DEV), inv.to(DEV), 1.0 / top)
     torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("N,top,E", [(1, 2, 4), (37, 3, 5), (64, 1, 2)])
+def test_moe_table_ffn_bf16(N, top, E):
+    W, ff, V = 96, 64, 50
+    dt = torch.bfloat16
+    h = rnd(N, W, dt=dt)
+    tok = torch.randint(0, V, (N,))
+    table = torch.stack([torch.randperm(E)[:top] for _ in range(V)]).int()
+    if N > 20:
+        table[:, 0] = 0                     # one crowded expert: > 16 rows
+    w_gu, w_down = rnd(E, 2 * ff, W, dt=dt, scale=0.1), \
+        rnd(E, W, ff, dt=dt, scale=0.1)
+    assert seq.moe_table_ffn_supported(h.to(DEV), top, ff)
+    got = seq.moe_table_ffn(h.to(DEV), tok.to(DEV), table.to(DEV),
+                            w_gu.to(DEV), w_down.to(DEV))
+    want = R.moe_table_ffn(h, tok, table, w_gu, w_down)
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=3e-2,
+                               atol=3e-2)
