@@ -44,6 +44,13 @@ void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
 void seq_moe_table_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
                        torch::Tensor tokens, torch::Tensor table,
                        torch::Tensor w_gu, torch::Tensor w_down);
+void seq_latent_attention_mfma(torch::Tensor out, torch::Tensor q,
+                               torch::Tensor cache, torch::Tensor page_table,
+                               torch::Tensor seq_of_tok,
+                               torch::Tensor positions, torch::Tensor tile_n0,
+                               torch::Tensor tile_cnt, int64_t rank,
+                               int64_t window, torch::Tensor sink,
+                               double scale, int64_t mode);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("seq_add_rmsnorm", &seq_add_rmsnorm,
@@ -63,6 +70,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "residual += scale * sum of a token's expert rows");
   m.def("seq_moe_table_ffn", &seq_moe_table_ffn,
         "table-routed expert feed-forward for decode-sized bf16 batches");
+  m.def("seq_latent_attention_mfma", &seq_latent_attention_mfma,
+        "windowed latent attention with sink on the matrix cores (bf16)");
   m.def("seq_delta_rule", &seq_delta_rule,
         "generalised delta rule scan (fp32 state, in place)");
   m.def("seq_ssm_scan", &seq_ssm_scan,

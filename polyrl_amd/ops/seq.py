@@ -177,13 +177,38 @@ def latent_kv_store(dkv, rank: int, norm_w, eps: float, positions, inv_freq,
                       slot_mapping)
 
 
+def attention_tiles(lens, device):
+    """Row tiles of a packed batch for the matrix-core attention kernel:
+    (first row, rows) per tile of at most 64 consecutive tokens of one
+    sequence, and the mode (1 when every sequence brings a single token:
+    a tile is then one token and up to 64 of its heads)."""
+    n0, cnt, at = [], [], 0
+    for n in lens:
+        for s in range(0, n, 64):
+            n0.append(at + s)
+            cnt.append(min(64, n - s))
+        at += n
+    mode = 1 if lens and max(lens) == 1 else 0
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    return i32(n0), i32(cnt), mode
+
+
 def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
                             positions, window: int, sink, scale: float,
-                            out_dtype) -> torch.Tensor:
+                            out_dtype, tiles=None) -> torch.Tensor:
     """Windowed attention of every row against its sequence's paged latent
     cache: score_j = (q_lat . c_j + q_rot . kr_j) * scale for
     0 <= pos - j < window; softmax whose denominator also holds exp(sink_h);
     returns sum_j p_j c_j, (N, H, rank).  All heads share the cache rows."""
+    row = q_lat.shape[2] + q_rot.shape[2]
+    if q_lat.is_cuda and tiles is not None and q_lat.shape[0] and \
+            q_lat.dtype == torch.bfloat16 and row % 8 == 0 and row <= 576:
+        out = torch.empty(q_lat.shape, dtype=out_dtype, device=q_lat.device)
+        _ext().seq_latent_attention_mfma(
+            out, torch.cat([q_lat, q_rot], -1), cache, page_table, seq_of_tok,
+            positions, tiles[0], tiles[1], q_lat.shape[2], window, sink,
+            scale, tiles[2])
+        return out
     if q_lat.is_cuda:
         out = torch.empty(q_lat.shape, dtype=out_dtype, device=q_lat.device)
         if q_lat.shape[0]:

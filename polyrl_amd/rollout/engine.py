@@ -783,7 +783,9 @@ class Engine:
             positions=i32(pos), seq_of_tok=i32(sot), cu_q=i32(cu),
             state_slot=i32(slots),
             slot_mapping=torch.cat(maps).to(dev),
-            page_table=self.kv.page_table(sids).to(dev)), cu
+            page_table=self.kv.page_table(sids).to(dev),
+            attn_tiles=ops.seq.attention_tiles(
+                [len(it[2]) for it in items], dev)), cu
 
     def _run_mixed(self, prefill_reqs, prefill_lens, decode_reqs):
         """One forward over prompt portions and single decode tokens

@@ -38,6 +38,7 @@ class HybridBatch:
     state_slot: torch.Tensor      # (B,)
     slot_mapping: torch.Tensor    # (N,) cache row of each token
     page_table: torch.Tensor      # (B, max_pages)
+    attn_tiles: Optional[tuple] = None   # ops.seq.attention_tiles(lens)
 
 
 _TUNED = False
@@ -201,7 +202,7 @@ class LatentAttnMixer(_Part):
         o_lat = seq.latent_window_attention(
             q_lat.contiguous(), q[:, :, s.dim:], rows, bt.page_table,
             bt.seq_of_tok, bt.positions, s.window, self.sink, s.scale,
-            h.dtype)
+            h.dtype, tiles=bt.attn_tiles)
         # ... and the value up-projection after the weighted sum
         o = torch.bmm(o_lat.transpose(0, 1),
                       self.uv.view(H, s.vdim, s.kv_rank).transpose(1, 2))

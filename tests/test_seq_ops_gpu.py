@@ -229,3 +229,41 @@ def test_moe_table_ffn_bf16(N, top, E):
     want = R.moe_table_ffn(h, tok, table, w_gu, w_down)
     torch.testing.assert_close(got.cpu().float(), want.float(), rtol=3e-2,
                                atol=3e-2)
+
+
+@pytest.mark.parametrize("H,R_,rd,window,lens,starts", [
+    (3, 64, 16, 5, [9, 1, 3], [0, 21, 6]),
+    (6, 40, 24, 40, [70, 2], [3, 90]),
+    (70, 256, 32, 33, [1, 1, 1], [0, 40, 131]),       # decode: heads as rows
+    (2, 512, 64, 100, [130], [17]),
+])
+def test_latent_attention_matrix_cores(H, R_, rd, window, lens, starts):
+    dt = torch.bfloat16
+    ps, pages = 16, 64
+    perm = torch.randperm(pages).tolist()
+    ptab, used = [], 0
+    for s, n in zip(starts, lens):
+        need = -(-(s + n) // ps)
+        ptab.append(perm[used:used + need] + [0] * (20 - need))
+        used += need
+    ptab_t = torch.tensor(ptab, dtype=torch.int32)
+    cache = rnd(pages, ps, R_ + rd, dt=dt)
+    pos, sot = [], []
+    for b, (s, n) in enumerate(zip(starts, lens)):
+        pos += list(range(s, s + n))
+        sot += [b] * n
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    N = len(pos)
+    q_lat, q_rot = rnd(N, H, R_, dt=dt, scale=0.3), rnd(N, H, rd, dt=dt)
+    sink = rnd(H)
+    sc = 1.0 / math.sqrt(R_ / 4 + rd)
+    want = R.latent_window_attention(q_lat, q_rot, cache, ptab_t, i32(sot),
+                                     i32(pos), window, sink, sc, dt)
+    tiles = seq.attention_tiles(lens, DEV)
+    assert tiles[2] == (1 if max(lens) == 1 else 0)
+    got = seq.latent_window_attention(
+        q_lat.to(DEV), q_rot.to(DEV), cache.to(DEV), ptab_t.to(DEV),
+        i32(sot).to(DEV), i32(pos).to(DEV), window, sink.to(DEV), sc, dt,
+        tiles=tiles)
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=3e-2,
+                               atol=3e-2)
