@@ -11,9 +11,15 @@
 // over rows (u^T S and S^T r, or S^T C) are two xor-shuffles inside the
 // 4-lane group, and a wave never synchronises with another.  The grid is
 // (sequence, head, 64-column block); HBM traffic is the state once in and
-// once out per portion plus the token inputs.  Inputs of token t+1 are
-// loaded before the arithmetic of token t so the dependent chain per token
-// is the VALU work only.  All state math is fp32 for bf16 or fp32 inputs.
+// once out per portion plus the token inputs.
+//
+// Per-token inputs of a lane's rows are contiguous and come in with 16-byte
+// loads when the layout allows (scalar loads otherwise); the inputs of token
+// t+1 are requested before the arithmetic of token t.  The delta rule's
+// decay and removal rate cost three exponentials per row: the 16 column
+// lanes of a row group would all compute the same ones, so each computes
+// one sixteenth and the group exchanges them by lane shuffles.
+// All state math is fp32 for bf16 or fp32 inputs.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -22,26 +28,69 @@
 constexpr int RG = 4;            // lanes sharing one column (row groups)
 constexpr int COLS_PER_WAVE = 16;
 
-// ------------------------------------------------------------- delta rule
+// dst[i] = p[i] for i < RPL (rows row0.. of `rows` in total); 16-byte loads
+// when the caller has checked alignment and rows == RG * RPL
 template <typename T, int RPL>
+DEV_INLINE void load_rows(float (&dst)[RPL], const T* p, int row0, int rows,
+                          bool vec) {
+  if (vec) {
+    if constexpr (sizeof(T) == 2 && RPL % 8 == 0) {
+#pragma unroll
+      for (int j = 0; j < RPL / 8; ++j) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + 8 * j);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[8 * j + e] = bf2f(v.v[e]);
+      }
+      return;
+    } else if constexpr (sizeof(T) == 4 && RPL % 4 == 0) {
+#pragma unroll
+      for (int j = 0; j < RPL / 4; ++j) {
+        const f32x4v v = *reinterpret_cast<const f32x4v*>(p + 4 * j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[4 * j + e] = v.v[e];
+      }
+      return;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) dst[i] = row0 + i < rows ? ldf(p + i) : 0.f;
+}
+
+// host check for load_rows' vector form: every lane's first row address
+// (view base + token row + column offset + head/group offset + row0) is
+// 16-byte aligned and no lane owns padding rows
+template <typename T>
+static bool rows_vectorizable(const torch::Tensor& t, long col_off, int rows,
+                              int rpl) {
+  const int per = 16 / (int)sizeof(T);
+  return rows == RG * rpl && rpl % per == 0 &&
+         ((uintptr_t)t.data_ptr() % 16 == 0) && t.stride(0) % per == 0 &&
+         col_off % per == 0 && rows % per == 0;
+}
+
+// ------------------------------------------------------------- delta rule
+template <int RPL>
 struct DeltaIn {
-  float r[RPL], k[RPL], wl[RPL], al[RPL];
+  static constexpr int NC = (RPL + 15) / 16;   // rows whose gates I compute
+  float r[RPL], k[RPL];
+  float wl[NC], al[NC];
   float v;
 };
 
 template <typename T, int RPL>
-DEV_INLINE void delta_load(DeltaIn<T, RPL>& in, const T* r, const T* k,
+DEV_INLINE void delta_load(DeltaIn<RPL>& in, const T* r, const T* k,
                            const T* v, const T* wl, const T* al, long ldr,
                            long ldk, long ldv, long ldw, long lda, long n,
-                           int hoff_k, int row0, int Dk, int vcol, bool colok) {
+                           int hoff_k, int row0, int Dk, int vcol, bool colok,
+                           int ci, bool vec) {
+  load_rows<T, RPL>(in.r, r + n * ldr + hoff_k + row0, row0, Dk, vec);
+  load_rows<T, RPL>(in.k, k + n * ldk + hoff_k + row0, row0, Dk, vec);
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) {
-    const int row = row0 + i;
-    const bool ok = row < Dk;
-    in.r[i] = ok ? ldf(r + n * ldr + hoff_k + row) : 0.f;
-    in.k[i] = ok ? ldf(k + n * ldk + hoff_k + row) : 0.f;
-    in.wl[i] = ok ? ldf(wl + n * ldw + hoff_k + row) : 0.f;
-    in.al[i] = ok ? ldf(al + n * lda + hoff_k + row) : 0.f;
+  for (int c = 0; c < DeltaIn<RPL>::NC; ++c) {
+    const int i = ci + 16 * c;
+    const bool ok = i < RPL && row0 + i < Dk;
+    in.wl[c] = ok ? ldf(wl + n * ldw + hoff_k + row0 + i) : 0.f;
+    in.al[c] = ok ? ldf(al + n * lda + hoff_k + row0 + i) : 0.f;
   }
   in.v = colok ? ldf(v + n * ldv + vcol) : 0.f;
 }
@@ -54,14 +103,16 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     long ldv, long ldw, long lda, const float* __restrict__ w0,
     const float* __restrict__ a_bias, float* __restrict__ state,
     const int* __restrict__ cu_q, const int* __restrict__ state_slot, int H,
-    int Dk, int Dv, float decay_scale, float key_eps) {
+    int Dk, int Dv, float decay_scale, float key_eps, bool vec) {
+  constexpr int NC = DeltaIn<RPL>::NC;
   const int cblocks = (Dv + 63) / 64;
   const int b = blockIdx.x / (H * cblocks);
   const int h = (blockIdx.x / cblocks) % H;
   const int cb = blockIdx.x % cblocks;
   const int lane = threadIdx.x & 63;
   const int wid = threadIdx.x >> 6;
-  const int col = cb * 64 + wid * COLS_PER_WAVE + lane / RG;
+  const int ci = lane / RG;                       // column index in the wave
+  const int col = cb * 64 + wid * COLS_PER_WAVE + ci;
   const int rg = lane % RG;
   const int row0 = rg * RPL;
   const bool colok = col < Dv;
@@ -71,25 +122,36 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   if (cb * 64 + wid * COLS_PER_WAVE >= Dv) return;
 
   float* S = state + (((long)state_slot[b] * H + h) * Dk) * Dv;
-  float s[RPL], w0r[RPL], abr[RPL];
+  float s[RPL], w0c[NC], abc[NC];
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
     const int row = row0 + i;
-    const bool ok = colok && row < Dk;
-    s[i] = ok ? S[(long)row * Dv + col] : 0.f;
-    w0r[i] = row < Dk ? w0[h * Dk + row] : 0.f;
-    abr[i] = row < Dk ? a_bias[h * Dk + row] : 0.f;
+    s[i] = (colok && row < Dk) ? S[(long)row * Dv + col] : 0.f;
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int i = ci + 16 * c;
+    const bool ok = i < RPL && row0 + i < Dk;
+    w0c[c] = ok ? w0[h * Dk + row0 + i] : 0.f;
+    abc[c] = ok ? a_bias[h * Dk + row0 + i] : 0.f;
   }
   const int hoff_k = h * Dk;
   const int vcol = h * Dv + col;
 
-  DeltaIn<T, RPL> cur, nxt;
+  DeltaIn<RPL> cur, nxt;
   delta_load<T, RPL>(cur, r, k, v, wl, al, ldr, ldk, ldv, ldw, lda, q0,
-                     hoff_k, row0, Dk, vcol, colok);
+                     hoff_k, row0, Dk, vcol, colok, ci, vec);
   for (int n = q0; n < q1; ++n) {
     if (n + 1 < q1)
       delta_load<T, RPL>(nxt, r, k, v, wl, al, ldr, ldk, ldv, ldw, lda, n + 1,
-                         hoff_k, row0, Dk, vcol, colok);
+                         hoff_k, row0, Dk, vcol, colok, ci, vec);
+    // my share of the gates: rows ci, ci+16, .. of this row group
+    float decm[NC], remm[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      decm[c] = expf(-decay_scale * sigmoidf_acc(cur.wl[c] + w0c[c]));
+      remm[c] = sigmoidf_acc(cur.al[c] + abc[c]);
+    }
     // unit key: |k|^2 over the head's Dk rows = sum over the 4 row groups
     float kk = 0.f;
 #pragma unroll
@@ -97,19 +159,16 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     kk = lanegroup_sum<RG>(kk);
     const float kinv = rsqrtf(kk + key_eps);
     float p = 0.f;
-    float u[RPL];
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
-      u[i] = cur.k[i] * kinv;
-      p += u[i] * s[i];
-    }
-    p = lanegroup_sum<RG>(p);
+    for (int i = 0; i < RPL; ++i) p += cur.k[i] * s[i];
+    p = lanegroup_sum<RG>(p) * kinv;               // u^T S (old state)
     float o = 0.f;
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-      const float dec = expf(-decay_scale * sigmoidf_acc(cur.wl[i] + w0r[i]));
-      const float rem = sigmoidf_acc(cur.al[i] + abr[i]);
-      s[i] = dec * s[i] - rem * u[i] * p + cur.k[i] * cur.v;
+      const int src = (i % 16) * RG + rg;          // lane that owns row i
+      const float dec = __shfl(decm[i / 16], src, WAVE_SIZE);
+      const float rem = __shfl(remm[i / 16], src, WAVE_SIZE);
+      s[i] = dec * s[i] - rem * (cur.k[i] * kinv) * p + cur.k[i] * cur.v;
       o += s[i] * cur.r[i];
     }
     o = lanegroup_sum<RG>(o);
@@ -131,7 +190,9 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
       w_lin.stride(0), a_lin.stride(0), w0.data_ptr<float>(),                \
       a_bias.data_ptr<float>(), state.data_ptr<float>(),                     \
       cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Dk, Dv,           \
-      (float)decay_scale, (float)key_eps)
+      (float)decay_scale, (float)key_eps,                                    \
+      rows_vectorizable<T>(r, 0, Dk, RPLV) &&                                \
+          rows_vectorizable<T>(k, 0, Dk, RPLV))
 
 void seq_delta_rule(torch::Tensor out, torch::Tensor r, torch::Tensor k,
                     torch::Tensor v, torch::Tensor w_lin, torch::Tensor a_lin,
@@ -184,14 +245,9 @@ template <typename T, int RPL>
 DEV_INLINE void ssm_load(SsmIn<RPL>& in, const T* xbc, long ldx, const T* dt,
                          long ldd, const T* z, long ldz, long n, int xcol,
                          int boff, int coff, int row0, int Ns, int h,
-                         bool colok) {
-#pragma unroll
-  for (int i = 0; i < RPL; ++i) {
-    const int row = row0 + i;
-    const bool ok = row < Ns;
-    in.Bv[i] = ok ? ldf(xbc + n * ldx + boff + row) : 0.f;
-    in.Cv[i] = ok ? ldf(xbc + n * ldx + coff + row) : 0.f;
-  }
+                         bool colok, bool vec) {
+  load_rows<T, RPL>(in.Bv, xbc + n * ldx + boff + row0, row0, Ns, vec);
+  load_rows<T, RPL>(in.Cv, xbc + n * ldx + coff + row0, row0, Ns, vec);
   in.x = colok ? ldf(xbc + n * ldx + xcol) : 0.f;
   in.z = colok ? ldf(z + n * ldz + xcol) : 0.f;
   in.dt = ldf(dt + n * ldd + h);
@@ -204,7 +260,8 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
     const T* __restrict__ z, long ldz, const float* __restrict__ dt_bias,
     const float* __restrict__ a_log, const float* __restrict__ d_skip,
     float* __restrict__ state, const int* __restrict__ cu_q,
-    const int* __restrict__ state_slot, int H, int Ns, int P, int G) {
+    const int* __restrict__ state_slot, int H, int Ns, int P, int G,
+    bool vec) {
   const int cblocks = (P + 63) / 64;
   const int b = blockIdx.x / (H * cblocks);
   const int h = (blockIdx.x / cblocks) % H;
@@ -237,11 +294,11 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
 
   SsmIn<RPL> cur, nxt;
   ssm_load<T, RPL>(cur, xbc, ldx, dt, ldd, z, ldz, q0, xcol, boff, coff, row0,
-                   Ns, h, colok);
+                   Ns, h, colok, vec);
   for (int n = q0; n < q1; ++n) {
     if (n + 1 < q1)
       ssm_load<T, RPL>(nxt, xbc, ldx, dt, ldd, z, ldz, n + 1, xcol, boff,
-                       coff, row0, Ns, h, colok);
+                       coff, row0, Ns, h, colok, vec);
     const float step = softplusf_acc(cur.dt + dtb);
     const float dec = expf(-A * step);
     const float sx = step * cur.x;
@@ -269,7 +326,8 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
       (const T*)dt.data_ptr(), dt.stride(0), (const T*)z.data_ptr(),         \
       z.stride(0), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),       \
       d_skip.data_ptr<float>(), state.data_ptr<float>(),                     \
-      cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Ns, P, (int)groups)
+      cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Ns, P,            \
+      (int)groups, rows_vectorizable<T>(xbc, (long)H * P, Ns, RPLV))
 
 void seq_ssm_scan(torch::Tensor out, torch::Tensor xbc, torch::Tensor dt,
                   torch::Tensor z, torch::Tensor dt_bias, torch::Tensor a_log,
