@@ -1,6 +1,12 @@
-"""Paged KV cache for the continuous-batching decoder.
+"""Paged caches and state slots for the continuous-batching decoder.
 
-Layout: per layer, K and V caches of shape (num_pages, page_size, Hk, D) bf16
+One page allocator (free list, per-sequence page lists, refcounts) serves
+two tensor layouts: K/V pages of the dense decoders and one latent row per
+token of the hybrid decoders' latent-attention layers.  Recurrent layers and
+stateful convolutions keep their per-sequence state in a fixed pool of
+slots (StateSlots), zeroed when handed out.
+
+K/V layout: per layer, K and V caches of shape (num_pages, page_size, Hk, D) bf16
 — the layout the HIP kernels (kv_cache.hip, attention_decode.hip) index.
 A simple free-list page allocator; per-sequence page lists grown on demand.
 Sized against a byte budget (288 GB HBM per MI355X; the scheduler decides the

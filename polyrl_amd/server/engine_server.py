@@ -307,7 +307,9 @@ def main():
     from ..models.registry import get_model_config
 
     p = argparse.ArgumentParser()
-    p.add_argument("--model", required=True)
+    p.add_argument("--model", required=True,
+                   help="registry name, or a checkpoint folder with "
+                        "config.json + *.safetensors")
     p.add_argument("--host", default="0.0.0.0")
     p.add_argument("--port", type=int, default=30001)
     p.add_argument("--dtype", default="bfloat16")
@@ -329,13 +331,26 @@ def main():
                         "(reference: allowed_sender_ips)")
     args = p.parse_args()
 
-    cfg = get_model_config(args.model)
     device = "cuda" if torch.cuda.is_available() else "cpu"
     dtype = getattr(torch, args.dtype) if device == "cuda" else torch.float32
-    engine = Engine(cfg, device=device, dtype=dtype,
-                    kv_bytes_budget=int(args.kv_gb * (1 << 30)),
-                    enable_radix_cache=args.radix_cache)
-    if args.load:
+    import os as _os0
+    if _os0.path.isdir(args.model) and args.load is None:
+        # a checkpoint folder: config.json picks the family, weights load
+        # by name (dense or hybrid decoders alike)
+        from ..rollout.loader import engine_from_dir
+        engine = engine_from_dir(args.model, device=device, dtype=dtype,
+                                 kv_bytes_budget=int(args.kv_gb * (1 << 30)),
+                                 enable_radix_cache=args.radix_cache)
+        cfg = engine.cfg
+        args.load = False
+    else:
+        cfg = get_model_config(args.model)
+        engine = Engine(cfg, device=device, dtype=dtype,
+                        kv_bytes_budget=int(args.kv_gb * (1 << 30)),
+                        enable_radix_cache=args.radix_cache)
+    if args.load is False:
+        pass
+    elif args.load:
         import os as _os
         if _os.path.isdir(args.load):
             # HF model dir (sharded safetensors): the engine's fused
@@ -351,6 +366,8 @@ def main():
         else:
             from safetensors.torch import load_file
             engine.model.load_state_dict(load_file(args.load), strict=False)
+    elif getattr(cfg, "is_hybrid", False):
+        engine.model.init_random(0)
     else:
         for _, t in engine.model._name_map.items():
             t.normal_(0, 0.02)
