@@ -321,10 +321,11 @@ class HybridLayer:
         self.side_norm = torch.empty(W, device=device, dtype=f32)
 
     def named(self, p: str) -> Dict[str, torch.Tensor]:
-        out = {p + "norm1": self.norm1, p + "canon1": self.canon,
-               p + "side.gate": self.side_gate,
-               p + "side.proj": self.side_proj,
-               p + "side.norm": self.side_norm}
+        out = {p + "norm1": self.norm1, p + "canon1": self.canon}
+        if self.side_gate.shape[0] > 0:
+            out.update({p + "side.gate": self.side_gate,
+                        p + "side.proj": self.side_proj,
+                        p + "side.norm": self.side_norm})
         out.update(self.mixer.named(p + "mix."))
         if self.ff is not None:
             out[p + "norm2"] = self.norm2
@@ -360,8 +361,10 @@ class HybridInferenceModel:
         self.lm_head = torch.empty(cfg.vocab_size, W, device=device,
                                    dtype=dtype)
         self._name_map: Dict[str, torch.Tensor] = {
-            "embed": self.embed, "side.embed": self.side_embed,
-            "final.norm": self.final_norm, "head": self.lm_head}
+            "embed": self.embed, "final.norm": self.final_norm,
+            "head": self.lm_head}
+        if cfg.token_side_dim > 0:
+            self._name_map["side.embed"] = self.side_embed
         for li, lw in enumerate(self.layers):
             self._name_map.update(lw.named(f"l{li}."))
         self.capture_layers: Optional[List[torch.Tensor]] = None
