@@ -191,29 +191,33 @@ void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
 }
 
 // ------------------------------------------------ grouped RMS norm (+gate)
-// out = y / rms_group(y) * w * (gate ? sigmoid(gate) : 1); one wave per
-// (row, group), groups of a row round-robin over the block's 4 waves.
-template <typename T>
+// out = y / rms_group(y) * w * (gate ? sigmoid(gate) : 1).  Small groups
+// (heads): one wave per (row, group), grid.y covers the groups four at a
+// time.  Large groups (BLOCK): the whole block reduces one (row, group).
+template <typename T, bool BLOCK>
 __global__ __launch_bounds__(256) void group_rmsnorm_kernel(
     T* __restrict__ out, const float* __restrict__ y,
     const float* __restrict__ w, const T* __restrict__ gate, long ldg, int D,
     int groups, float eps) {
+  __shared__ float red[8];
   const long row = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wid = threadIdx.x >> 6;
   const int gs = D / groups;
-  for (int g = wid; g < groups; g += 4) {
-    const float* yr = y + row * D + (long)g * gs;
-    float ss = 0.f;
-    for (int i = lane; i < gs; i += 64) ss += yr[i] * yr[i];
-    ss = wave_reduce_sum(ss);
-    const float inv = rsqrtf(ss / gs + eps);
-    for (int i = lane; i < gs; i += 64) {
-      const int c = g * gs + i;
-      float v = yr[i] * inv * w[c];
-      if (gate) v *= sigmoidf_acc(ldf(gate + row * ldg + c));
-      stf(out + row * D + c, v);
-    }
+  const int g = BLOCK ? blockIdx.y : blockIdx.y * 4 + wid;
+  if (g >= groups) return;                  // wave-uniform (block-uniform)
+  const int t0 = BLOCK ? threadIdx.x : lane;
+  const int step = BLOCK ? 256 : 64;
+  const float* yr = y + row * D + (long)g * gs;
+  float ss = 0.f;
+  for (int i = t0; i < gs; i += step) ss += yr[i] * yr[i];
+  ss = BLOCK ? block_reduce_sum<4>(ss, red) : wave_reduce_sum(ss);
+  const float inv = rsqrtf(ss / gs + eps);
+  for (int i = t0; i < gs; i += step) {
+    const int c = g * gs + i;
+    float v = yr[i] * inv * w[c];
+    if (gate) v *= sigmoidf_acc(ldf(gate + row * ldg + c));
+    stf(out + row * D + c, v);
   }
 }
 
@@ -233,10 +237,22 @@ void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
   }
   if (y.size(0) == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
-  SEQ_DISPATCH_T(out.scalar_type(), { hipLaunchKernelGGL((group_rmsnorm_kernel<T>), dim3(y.size(0)), dim3(256), 0, stream, 
-      (T*)out.data_ptr(), y.data_ptr<float>(), weight.data_ptr<float>(),
-      has_g ? (const T*)gate.data_ptr() : nullptr, has_g ? gate.stride(0) : 0,
-      D, (int)groups, (float)eps); });
+  const bool big = D / groups >= 512;
+  const dim3 grid(y.size(0), big ? groups : (groups + 3) / 4);
+  SEQ_DISPATCH_T(out.scalar_type(), {
+    if (big)
+      hipLaunchKernelGGL((group_rmsnorm_kernel<T, true>), grid, dim3(256), 0,
+          stream, (T*)out.data_ptr(), y.data_ptr<float>(),
+          weight.data_ptr<float>(),
+          has_g ? (const T*)gate.data_ptr() : nullptr,
+          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps);
+    else
+      hipLaunchKernelGGL((group_rmsnorm_kernel<T, false>), grid, dim3(256), 0,
+          stream, (T*)out.data_ptr(), y.data_ptr<float>(),
+          weight.data_ptr<float>(),
+          has_g ? (const T*)gate.data_ptr() : nullptr,
+          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps);
+  });
   HIP_CHECK_KERNEL();
 }
 

@@ -797,7 +797,16 @@ class Engine:
         for r in decode_reqs:
             items.append((r, r.seq_len - 1, [r.output_ids[-1]]))
         bt, cu = self._hybrid_batch(items)
-        res = self.model.forward_batch(bt, self.kv, self.states)
+        # pure decode steps recur with few distinct shapes: worth the pinned
+        # per-shape GEMM algorithms; ragged prompt portions are not
+        from . import hybrid_model
+        hybrid_model.set_tuned_products(
+            not prefill_reqs and _tuned_decode_enabled()
+            and ops.extension_loaded())
+        try:
+            res = self.model.forward_batch(bt, self.kv, self.states)
+        finally:
+            hybrid_model.set_tuned_products(False)
         rows, reqs = [], []
         for i, (r, take) in enumerate(zip(prefill_reqs, prefill_lens)):
             r.prefill_pos += take
