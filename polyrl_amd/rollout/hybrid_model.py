@@ -55,7 +55,8 @@ def set_tuned_products(on: bool) -> None:
 def _mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """y = x @ w.T (vendor matrix product, fp32 accumulation)."""
     if _TUNED and x.is_cuda and x.dtype == torch.bfloat16 \
-            and x.shape[0] <= 512 and x.is_contiguous():
+            and x.shape[0] <= 512 and x.is_contiguous() \
+            and w.shape[0] >= 64 and w.shape[1] >= 64:
         return ops.tuned_mm_nt(x, w)
     return x @ w.t()
 

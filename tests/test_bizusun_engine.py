@@ -342,7 +342,7 @@ def test_folder_loader_and_trace_replay(target, tmp_path, monkeypatch, capsys):
     close(g2, wa[12:13], target, "step 2")
 
 
-@pytest.mark.parametrize("target", [CPU, GPU32])
+@pytest.mark.parametrize("target", TARGETS)
 def test_greedy_generation_through_the_scheduler(target):
     """Engine.generate: admission, chunked prompts (token budget of 8),
     mixed steps, sampling at temperature 0, slots released at the end."""
@@ -359,7 +359,9 @@ def test_greedy_generation_through_the_scheduler(target):
         for got_tok in o.output_ids:
             logits = O.forward(FULL, W, ids)[-1]
             top2 = logits.topk(2).values
-            if float(top2[0] - top2[1]) > 1e-3:     # skip near ties
+            tie = 1e-3 if target[1] == torch.float32 else \
+                0.25 * float(logits.std())
+            if float(top2[0] - top2[1]) > tie:      # skip near ties
                 assert got_tok == int(logits.argmax())
             ids.append(got_tok)
         assert len(o.output_ids) == 5 and o.finish_reason == "length"
