@@ -12,7 +12,8 @@
 // the rows are up to 64 heads of one token.  QK^T and P.V run on
 // v_mfma_f32_16x16x32_bf16 (A = Q rows / P, B = K^T / V from LDS, fp32
 // accumulators); the softmax is online per row in fp32 and starts from the
-// sink (m = sink_h, l = 1, O = 0).  K-tile bytes are XOR-swizzled by row
+// sink (m = sink_h, l = 1, O = 0).  The next tile's rows are fetched into
+// registers while the current tile is multiplied.  K-tile bytes are XOR-swizzled by row
 // inside each 64-byte chunk (a row is a whole number of such chunks) so the
 // 16 rows of a B-fragment read spread over the banks.
 #include <torch/extension.h>
@@ -94,21 +95,42 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
   for (int nt = 0; nt < NVT; ++nt) o_acc[nt] = {0.f, 0.f, 0.f, 0.f};
 
-  for (int t0 = kmin; t0 <= pmax; t0 += AKV) {
-    // ---- stage 32 cached rows (zero past the row end / the last key) ----
-    for (int v = threadIdx.x; v < AKV * KS * 4; v += 256) {
+  // global -> register prefetch of one tile (this thread's 16-byte vectors;
+  // zero past the row end / the last key), issued one tile ahead so its
+  // latency hides behind the previous tile's matrix work
+  constexpr int NV = (AKV * KS * 4 + 255) / 256;
+  i32x4_t pre[NV];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * 256;
       const int kr = v / (KS * 4);
       const int col = (v % (KS * 4)) * 8;
       const int j = t0 + kr;
-      i32x4_t val = {0, 0, 0, 0};
-      if (j <= pmax && col < row) {
+      const i32x4_t z = {0, 0, 0, 0};
+      pre[i] = z;
+      if (v < AKV * KS * 4 && j <= pmax && col < row) {
         const long slot = (long)ptab[j / page_size] * page_size + j % page_size;
-        val = *reinterpret_cast<const i32x4_t*>(cache + slot * row + col);
+        pre[i] = *reinterpret_cast<const i32x4_t*>(cache + slot * row + col);
       }
-      *reinterpret_cast<i32x4_t*>(reinterpret_cast<char*>(Ks) +
-                                  tile_off<KS>(kr, col * 2)) = val;
+    }
+  };
+  fetch(kmin);
+
+  for (int t0 = kmin; t0 <= pmax; t0 += AKV) {
+    // ---- registers -> swizzled LDS tile, then request the next tile ------
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * 256;
+      if (v < AKV * KS * 4) {
+        const int kr = v / (KS * 4);
+        const int col = (v % (KS * 4)) * 8;
+        *reinterpret_cast<i32x4_t*>(reinterpret_cast<char*>(Ks) +
+                                    tile_off<KS>(kr, col * 2)) = pre[i];
+      }
     }
     __syncthreads();
+    if (t0 + AKV <= pmax) fetch(t0 + AKV);
 
     // ---- S (16 rows x 32 keys) = Q K^T ----------------------------------
     f32x4_t c[2];
