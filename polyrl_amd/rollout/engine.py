@@ -518,6 +518,16 @@ class Engine:
         257-284 — used when trainer and rollout time-share a tight GPU).
         Requires an idle engine; resume_memory() reallocates."""
         assert not self.has_work(), "release_memory needs an idle engine"
+        if self.hybrid:
+            # idle engine: no live pages or slots, so dropping the tensors
+            # loses nothing; resume_memory() rebuilds both pools
+            self._kv_shape = (self.kv.num_pages, self.kv.page_size)
+            self.kv.rows = {}
+            self.states.tensors = {}
+            self._kv_released = True
+            if str(self.device).startswith("cuda"):
+                torch.cuda.empty_cache()
+            return
         self._kv_shape = (self.kv.num_layers, self.kv.num_kv_heads,
                           self.kv.head_dim, self.kv.num_pages,
                           self.kv.page_size)
@@ -538,6 +548,14 @@ class Engine:
 
     def resume_memory(self):
         if not getattr(self, "_kv_released", False):
+            return
+        if self.hybrid:
+            P, ps = self._kv_shape
+            self.kv = PagedLatentCache(self.model.cache_row_dims(), P, ps,
+                                       dtype=self.dtype, device=self.device)
+            self.states = StateSlots(self.model.state_shapes(),
+                                     self.max_running, device=self.device)
+            self._kv_released = False
             return
         L, Hk, D, P, ps = self._kv_shape
         self.kv = PagedKVCache(L, Hk, D, P, ps, dtype=self.dtype,

@@ -367,3 +367,14 @@ def test_greedy_generation_through_the_scheduler(target):
         assert len(o.output_ids) == 5 and o.finish_reason == "length"
     assert e.kv.free_pages == e.kv.num_pages
     assert e.states.free_slots == e.states.num_slots
+
+
+def test_release_and_resume_memory():
+    W = O.random_weights(FULL, seed=43)
+    e = engine(FULL, W, CPU)
+    t = toks(9, seed=90)
+    a = run(e, "a", t)
+    e.release_memory()
+    assert not e.kv.rows and not e.states.tensors
+    e.resume_memory()
+    torch.testing.assert_close(run(e, "b", t), a)
