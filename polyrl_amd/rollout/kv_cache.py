@@ -10,7 +10,7 @@ K/V layout: per layer, K and V caches of shape (num_pages, page_size, Hk, D) bf1
 — the layout the HIP kernels (kv_cache.hip, attention_decode.hip) index.
 A simple free-list page allocator; per-sequence page lists grown on demand.
 Sized against a byte budget (288 GB HBM per MI355X; the scheduler decides the
-split between weights / KV / activations — SURVEY.md §5.9).
+split between weights / KV / activations).
 """
 from __future__ import annotations
 
@@ -31,8 +31,8 @@ class PageAllocator:
         self._free: List[int] = list(range(num_pages - 1, -1, -1))
         self._seq_pages: Dict[int, List[int]] = {}
         self._seq_len: Dict[int, int] = {}
-        # page refcounts for prefix sharing (radix-cache capability,
-        # SURVEY.md §2.4.3): n samples of one prompt share its full pages
+        # page refcounts for prefix sharing (radix-cache capability):
+        # n samples of one prompt share its full pages
         self._ref: Dict[int, int] = {}
 
     # ------------------------------------------------------------- accounting
@@ -271,8 +271,7 @@ class _RadixNode:
 
 class RadixCache:
     """Cross-request KV prefix cache (the SGLang radix-cache capability the
-    reference relies on for shared system prompts / multi-turn reuse —
-    SURVEY.md §2.2.2 kernel-suite row, §2.4.3).
+    reference relies on for shared system prompts / multi-turn reuse).
 
     Page-granular trie: each node is exactly ``page_size`` tokens pinning one
     KV page (+1 on the allocator refcount).  A new request walks the trie
