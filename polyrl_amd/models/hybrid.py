@@ -69,11 +69,94 @@ class LatentAttnSpec:
 
 
 @dataclass
+class RopeSpec:
+    """Rotate-half rotary positions on the first ``dims`` entries of every
+    head.  ``factor`` > 1 switches on YaRN: pairs that turn fewer than
+    ``slow`` times within ``original`` positions have their frequency divided
+    by ``factor``, pairs that turn more than ``fast`` times keep it, a linear
+    ramp joins the two, and cos/sin are scaled by ``amp_slope*ln(factor)+1``."""
+    dims: int
+    base: float = 10000.0
+    factor: float = 1.0
+    original: float = 0.0
+    fast: float = 32.0
+    slow: float = 1.0
+    amp_slope: float = 0.1
+
+    def inv_freq_and_amp(self):
+        """(per-pair frequencies as Python floats, cos/sin amplitude)."""
+        dims, half = self.dims, self.dims // 2
+        f = [self.base ** (-2.0 * i / dims) for i in range(half)]
+        if self.factor == 1.0 or self.original <= 0:
+            return f, 1.0
+
+        def pair_of(turns):
+            return dims * math.log(self.original / (2 * math.pi * turns)) / \
+                (2 * math.log(self.base))
+        lo = max(math.floor(pair_of(self.fast)), 0)
+        hi = min(math.ceil(pair_of(self.slow)), dims - 1)
+        out = []
+        for i in range(half):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(f[i] / self.factor * ramp + f[i] * (1.0 - ramp))
+        return out, self.amp_slope * math.log(self.factor) + 1.0
+
+
+@dataclass
+class WindowAttnSpec:
+    """Grouped-query softmax attention over a sliding window of a paged
+    K/V cache.  Optional parts, each a parameter: rotary positions
+    (``rope``), first tokens that stay visible (``keep_first``), RMS norms
+    over the whole query / key projection (``qk_norm``), values taken from
+    the raw key projection (``values_from_keys``: no value matrix), one
+    sigmoid output gate per head (``head_gate``), and a learned bias per
+    (distance bucket, head) added to the scaled scores (``bias_far`` > 0:
+    the bucket of distance n is n below half the table's rows, logarithmic
+    steps up to ``bias_far`` above)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int
+    scale: float
+    keep_first: int = 0
+    rope: Optional[RopeSpec] = None
+    qk_norm: bool = False
+    values_from_keys: bool = False
+    head_gate: bool = False
+    bias_far: float = 0.0
+    bias_rows: Optional[int] = None       # rows of the table; None = tensor
+    kind: str = "attention"
+
+    def bucket_of_distance(self) -> List[int]:
+        """Bias-table row for every distance 0 .. window-1."""
+        rows, far = int(self.bias_rows), float(self.bias_far)
+        half = rows // 2
+        out = []
+        for n in range(self.window):
+            if n < half:
+                out.append(n)
+            else:
+                out.append(min(rows - 1, half + int(math.floor(
+                    math.log(n / half) / math.log(far / half)
+                    * (rows - half)))))
+        return out
+
+
+@dataclass
 class FFSpec:
-    kind: str                 # dense | moe
+    kind: str                 # dense | moe | routed_moe
     ff: int                   # hidden size (of one expert for moe)
     experts: int = 0
     top: int = 0
+    # routed_moe: softmax router with a selection-only correction, experts
+    # in equal groups of neighbours of which the best ``group_keep`` stay
+    # eligible, trailing identity experts, an always-on shared expert
+    identity: int = 0
+    group_count: int = 1
+    group_keep: int = 1
+    shared_ff: int = 0
+    weight_eps: float = 1e-20
 
 
 @dataclass
@@ -93,6 +176,15 @@ class HybridConfig:
     token_side_dim: int = 0
     logit_scale: float = 1.0
     max_position_embeddings: int = 1 << 20   # no learned positions: a fence
+    # "canon": norm -> convolution -> mixer, norm -> ff, token-side input
+    # (scalar norm weights).  "sandwich": x += norm(mixer(norm(x))),
+    # x += norm(ff(norm(x))) with per-channel weights stored as offsets
+    # from ``norm_offset``.
+    layer_style: str = "canon"
+    norm_offset: float = 0.0
+    # layers [start, stop) run ``times`` times in a row with the same
+    # weights; every pass owns its cache rows and state
+    loop: Optional[tuple] = None
 
     # the engine's generic accessors
     @property
@@ -102,6 +194,15 @@ class HybridConfig:
     @property
     def is_hybrid(self) -> bool:
         return True
+
+    def run_order(self) -> List[int]:
+        """Layer index of every layer run, in execution order.  Caches and
+        states are keyed by the run's place in this list."""
+        n = len(self.layers)
+        if not self.loop or self.loop[2] <= 1:
+            return list(range(n))
+        a, b, t = self.loop
+        return list(range(a)) + list(range(a, b)) * t + list(range(b, n))
 
     def cache_owner(self, li: int) -> Optional[int]:
         """Layer whose latent cache layer ``li`` reads (itself unless it
@@ -127,8 +228,28 @@ class HybridConfig:
             if m.kind == "mamba2":
                 assert m.heads % m.groups == 0
                 assert m.inner % m.norm_groups == 0
+            if m.kind == "attention":
+                assert m.heads % m.kv_heads == 0 and m.window >= 1
+                if m.rope is not None:
+                    assert m.rope.dims % 2 == 0 and m.rope.dims <= m.dim
+                if m.bias_far > 0 and m.keep_first > 0:
+                    raise ValueError(f"layer {li}: the distance bias covers "
+                                     "the window only (no kept first tokens)")
             if L.ff is not None and L.ff.kind == "moe":
                 assert 0 < L.ff.top <= L.ff.experts
+            if L.ff is not None and L.ff.kind == "routed_moe":
+                f = L.ff
+                total = f.experts + f.identity
+                assert total % f.group_count == 0
+                assert 0 < f.group_keep <= f.group_count
+                assert 0 < f.top <= f.group_keep * (total // f.group_count)
+        if self.loop is not None:
+            a, b, t = self.loop
+            assert 0 <= a <= b <= len(self.layers) and t >= 1
+            if any(getattr(L.mixer, "kv_from", None) is not None
+                   for L in self.layers):
+                raise ValueError("shared caches and looped layers do not "
+                                 "combine")
         return self
 
 
@@ -252,6 +373,147 @@ def bizusun_preset(width: int, layers: int, vocab: int = 32000,
                         logit_scale=1.0).validate()
 
 
+def _window_attn_from_json(kind: str, m: dict) -> WindowAttnSpec:
+    """Kuforax mixers: 'attention' (rotary, kept first tokens, whole-row
+    query/key norms, values = raw keys, per-head gate) and 'attention_2'
+    (distance-bucket bias, separate values, no rotation)."""
+    mask = m["mask"]
+    common = dict(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                  dim=int(m["dim"]), vdim=int(m["vdim"]),
+                  window=int(mask["size"]), scale=float(m["scale"]))
+    if kind == "attention":
+        rot = m.get("rot")
+        rope = None
+        if rot and int(rot.get("dims", 0)) > 0:
+            sc = rot.get("scaling") or {}
+            rope = RopeSpec(dims=int(rot["dims"]), base=float(rot["base"]),
+                            factor=float(sc.get("factor", 1.0)),
+                            original=float(sc.get("original", 0.0)),
+                            fast=float(sc.get("fast", 32.0)),
+                            slow=float(sc.get("slow", 1.0)))
+        if common["vdim"] != common["dim"]:
+            raise ValueError("values taken from keys need vdim == dim")
+        return WindowAttnSpec(**common, rope=rope,
+                              keep_first=int(mask.get("keep_first", 0)),
+                              qk_norm=True, values_from_keys=True,
+                              head_gate=True)
+    return WindowAttnSpec(**common, bias_far=float(m["bias_max"]))
+
+
+def _routed_ff_from_json(f: Optional[dict]) -> Optional[FFSpec]:
+    if f is None:
+        return None
+    if f["kind"] != "moe":
+        raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+    r = f["router"]
+    g = r.get("groups") or {}
+    shared = f.get("shared") or {}
+    return FFSpec(kind="routed_moe", ff=int(f["expert"]["ff"]),
+                  experts=int(r["experts"]), top=int(r["top"]),
+                  identity=int(r.get("identity", 0)),
+                  group_count=int(g.get("count", 1)),
+                  group_keep=int(g.get("keep", 1)),
+                  shared_ff=int(shared.get("ff", 0)))
+
+
+def kuforax_config_from_json(d: dict) -> HybridConfig:
+    """Read a Kuforax ``config.json`` (already parsed)."""
+    layers = []
+    for L in d["layers"]:
+        if L["type"] not in ("attention", "attention_2"):
+            raise ValueError(f"unknown mixer type {L['type']!r}")
+        layers.append(HybridLayerSpec(
+            _window_attn_from_json(L["type"], L["mixer"]),
+            _routed_ff_from_json(L.get("mlp"))))
+    loop = d.get("loop")
+    return HybridConfig(
+        arch="kuforax", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), layers=layers,
+        norm_eps=float(d["norm"]["eps"]), canon_taps=1, token_side_dim=0,
+        layer_style="sandwich", norm_offset=1.0,
+        loop=None if not loop else (int(loop["start"]), int(loop["stop"]),
+                                    int(loop["times"]))).validate()
+
+
+def kuforax_config_to_json(cfg: HybridConfig) -> dict:
+    """Inverse of :func:`kuforax_config_from_json` (checkpoint export)."""
+    layers = []
+    for L in cfg.layers:
+        m = L.mixer
+        mj = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+              "vdim": m.vdim, "scale": m.scale, "mask": {"size": m.window}}
+        if m.bias_far > 0:
+            kind = "attention_2"
+            mj["bias_max"] = m.bias_far
+        else:
+            kind = "attention"
+            mj["mask"]["keep_first"] = m.keep_first
+            if m.rope is not None:
+                r = m.rope
+                mj["rot"] = {"base": r.base, "dims": r.dims}
+                if r.factor != 1.0:
+                    mj["rot"]["scaling"] = {
+                        "factor": r.factor, "original": r.original,
+                        "fast": r.fast, "slow": r.slow}
+        fj = None
+        if L.ff is not None:
+            f = L.ff
+            fj = {"kind": "moe", "expert": {"ff": f.ff},
+                  "router": {"experts": f.experts, "top": f.top,
+                             "identity": f.identity,
+                             "groups": {"count": f.group_count,
+                                        "keep": f.group_keep}}}
+            if f.shared_ff:
+                fj["shared"] = {"ff": f.shared_ff}
+        layers.append({"type": kind, "mixer": mj, "mlp": fj})
+    out = {"architecture": "Kuforax", "vocab": cfg.vocab_size,
+           "width": cfg.hidden_size, "layers": layers,
+           "norm": {"eps": cfg.norm_eps}}
+    if cfg.loop is not None:
+        out["loop"] = {"start": cfg.loop[0], "stop": cfg.loop[1],
+                       "times": cfg.loop[2]}
+    return out
+
+
+def kuforax_preset(width: int, layers: int, vocab: int = 32000,
+                   heads: int = 16, kv_heads: int = 4, experts: int = 16,
+                   top: int = 2, identity: int = 2, expert_ff: int = 0,
+                   shared_ff: int = 0, window: int = 1024,
+                   keep_first: int = 4, bias_every: int = 4,
+                   loop: Optional[tuple] = None) -> HybridConfig:
+    """A Kuforax stack of realistic layer sizes (random weights): every
+    ``bias_every``-th layer uses the distance-bias attention, the others
+    the rotary one; routed experts with a shared expert in every layer."""
+    hd = width // heads
+    expert_ff = expert_ff or max(64, width // 64 * 64)
+    shared_ff = shared_ff or expert_ff
+    total = experts + identity
+    groups = 2 if total % 2 == 0 and total // 2 >= top else 1
+    out = []
+    for li in range(layers):
+        if bias_every and li % bias_every == bias_every - 1:
+            mixer = WindowAttnSpec(heads=heads, kv_heads=kv_heads, dim=hd,
+                                   vdim=hd, window=window,
+                                   scale=1.0 / math.sqrt(hd),
+                                   bias_far=float(window), bias_rows=32)
+        else:
+            mixer = WindowAttnSpec(
+                heads=heads, kv_heads=kv_heads, dim=hd, vdim=hd,
+                window=window, scale=1.0 / math.sqrt(hd),
+                keep_first=keep_first,
+                rope=RopeSpec(dims=hd // 2, base=10000.0, factor=4.0,
+                              original=4096.0),
+                qk_norm=True, values_from_keys=True, head_gate=True)
+        ff = FFSpec("routed_moe", expert_ff, experts, top, identity=identity,
+                    group_count=groups, group_keep=1 if groups > 1 else 1,
+                    shared_ff=shared_ff)
+        out.append(HybridLayerSpec(mixer, ff))
+    return HybridConfig(arch="kuforax", vocab_size=vocab, hidden_size=width,
+                        layers=out, norm_eps=1e-5, canon_taps=1,
+                        token_side_dim=0, layer_style="sandwich",
+                        norm_offset=1.0, loop=loop).validate()
+
+
 def read_config_dir(path: str):
     """Model config from a checkpoint folder's ``config.json``.  The
     ``architecture`` key names the family; HF-style folders
@@ -261,6 +523,8 @@ def read_config_dir(path: str):
     arch = d.get("architecture")
     if arch == "Bizusun":
         return bizusun_config_from_json(d)
+    if arch == "Kuforax":
+        return kuforax_config_from_json(d)
     mt = d.get("model_type")
     if mt in ("llama", "qwen2"):
         from .registry import DecoderConfig

@@ -97,8 +97,18 @@ MODEL_CONFIGS = {
 
 
 def _hybrid_presets():
-    from .hybrid import bizusun_preset
+    from .hybrid import bizusun_preset, kuforax_preset
     return {
+        # tiny looped stack for CPU unit tests / fast GPU smoke
+        "kuforax-debug": lambda: kuforax_preset(
+            width=64, layers=3, vocab=300, heads=4, kv_heads=2, experts=6,
+            top=2, identity=2, expert_ff=32, shared_ff=48, window=24,
+            keep_first=3, bias_every=3, loop=(1, 3, 2)),
+        # layer sizes of a ~1B-class model (bench: beside llama3-1b)
+        "kuforax-1b": lambda: kuforax_preset(
+            width=2048, layers=16, vocab=128256, heads=32, kv_heads=8,
+            experts=16, top=2, identity=2, expert_ff=2560, shared_ff=2560,
+            window=1024, keep_first=4),
         # tiny hybrid for CPU unit tests / fast GPU smoke
         "bizusun-debug": lambda: bizusun_preset(
             width=64, layers=5, vocab=300, heads=2, experts=4, top=2,

@@ -41,15 +41,16 @@ def _ext():
 
 def add_rmsnorm_f32res(res: torch.Tensor, y: Optional[torch.Tensor],
                        weight: torch.Tensor, eps: float,
-                       out_dtype: torch.dtype) -> torch.Tensor:
-    """res (N, D) fp32 += y in place, then RMS-norm(res) * weight -> out_dtype.
-    ``weight`` holds one number (for all coordinates) or D."""
+                       out_dtype: torch.dtype,
+                       offset: float = 0.0) -> torch.Tensor:
+    """res (N, D) fp32 += y in place, then RMS-norm(res) * (offset + weight)
+    -> out_dtype.  ``weight`` holds one number (for all coordinates) or D."""
     if res.is_cuda:
         out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
         _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
-                               weight, eps, 0)
+                               weight, eps, 0, offset, torch.Tensor())
         return out
-    return R.add_rmsnorm_f32res(res, y, weight, eps, out_dtype)
+    return R.add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset)
 
 
 def residual_add_cast(res: torch.Tensor, y: Optional[torch.Tensor],
@@ -61,18 +62,35 @@ def residual_add_cast(res: torch.Tensor, y: Optional[torch.Tensor],
         out = res if out_dtype == torch.float32 else \
             torch.empty(res.shape, dtype=out_dtype, device=res.device)
         _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
-                               torch.Tensor(), 0.0, 1)
+                               torch.Tensor(), 0.0, 1, 0.0, torch.Tensor())
         return out
     return R.residual_add_cast(res, y, out_dtype)
 
 
 def add_scaled_unit_rms(res: torch.Tensor, y: torch.Tensor,
-                        weight: torch.Tensor, eps: float) -> None:
-    """res += y / rms(y) * weight, in place (weight (D,) fp32)."""
+                        weight: torch.Tensor, eps: float,
+                        offset: float = 0.0) -> None:
+    """res += y / rms(y) * (offset + weight), in place (weight (D,) fp32)."""
     if res.is_cuda:
-        _ext().seq_add_rmsnorm(res, res, y, weight, eps, 2)
+        _ext().seq_add_rmsnorm(res, res, y, weight, eps, 2, offset,
+                               torch.Tensor())
         return
-    R.add_scaled_unit_rms(res, y, weight, eps)
+    R.add_scaled_unit_rms(res, y, weight, eps, offset)
+
+
+def add_unit_rms_then_norm(res: torch.Tensor, y: torch.Tensor,
+                           w_post: torch.Tensor, w_next: torch.Tensor,
+                           eps: float, out_dtype: torch.dtype,
+                           offset: float = 0.0) -> torch.Tensor:
+    """The joint between two normed sublayers in one pass over the row:
+    res += y / rms(y) * (offset + w_post) in place, then returns
+    res / rms(res) * (offset + w_next) as out_dtype."""
+    if res.is_cuda:
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        _ext().seq_add_rmsnorm(out, res, y, w_post, eps, 3, offset, w_next)
+        return out
+    return R.add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype,
+                                    offset)
 
 
 def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,
@@ -219,6 +237,132 @@ def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
     return R.latent_window_attention(q_lat, q_rot, cache, page_table,
                                      seq_of_tok, positions, window, sink,
                                      scale, out_dtype)
+
+
+def gqa_prepare_store(q, k, v, q_norm, k_norm, eps: float, inv_freq,
+                      amp: float, positions, cache, slot_mapping, H: int,
+                      G: int, D: int, Dv: int) -> torch.Tensor:
+    """Queries and cache rows of grouped-query attention from a step's
+    projections (column slices allowed).  Optional RMS norm over the WHOLE
+    query row and the whole key row (weights q_norm / k_norm), then
+    rotate-half RoPE on the first 2*len(inv_freq) entries of every head with
+    angle fp32(position)*inv_freq and cos/sin scaled by ``amp``.  The cache
+    row of a token, (pages, page_size, G*D + G*Dv) at slot_mapping[n], is
+    [keys (normed, rotated) | values]; values are ``v`` or, when ``v`` is
+    None, the key projection as it came in.  Returns the queries (N, H*D)."""
+    if q.is_cuda:
+        out = torch.empty(q.shape[0], H * D, dtype=q.dtype, device=q.device)
+        if q.shape[0]:
+            e = torch.Tensor()
+            _ext().seq_gqa_prepare_store(
+                out, q, k, v if v is not None else e,
+                q_norm if q_norm is not None else e,
+                k_norm if k_norm is not None else e, eps,
+                inv_freq if inv_freq is not None else e, amp, positions,
+                cache, slot_mapping, H, G, D, Dv)
+        return out
+    return R.gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp,
+                               positions, cache, slot_mapping, H, G, D, Dv)
+
+
+def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
+                         G: int, D: int, Dv: int, window: int,
+                         keep_first: int, rel, dist_bucket, gate,
+                         scale: float, out_dtype, tiles=None) -> torch.Tensor:
+    """Softmax attention of every row against its sequence's paged K/V rows
+    (layout of :func:`gqa_prepare_store`).  Row at position p sees key j if
+    j <= p and (p - j < window or j < keep_first).  score = q.k * scale
+    [+ rel[dist_bucket[p - j], head]]; ``gate`` (N, H) multiplies head h's
+    output by sigmoid(gate[n, h]).  Query head h reads key/value head
+    h // (H // G).  Returns (N, H*Dv)."""
+    if q.is_cuda:
+        out = torch.empty(q.shape[0], H * Dv, dtype=out_dtype,
+                          device=q.device)
+        if q.shape[0]:
+            e = torch.Tensor()
+            args = (cache, page_table, seq_of_tok, positions, H, G, D, Dv,
+                    window, keep_first, rel if rel is not None else e,
+                    dist_bucket if dist_bucket is not None else e,
+                    gate if gate is not None else e, scale)
+            if tiles is not None and gqa_mfma_supported(q, D, Dv):
+                _ext().seq_gqa_window_attention_mfma(out, q, tiles[0],
+                                                     tiles[1], *args)
+            else:
+                _ext().seq_gqa_window_attention(out, q, *args)
+        return out
+    return R.gqa_window_attention(q, cache, page_table, seq_of_tok, positions,
+                                  H, G, D, Dv, window, keep_first, rel,
+                                  dist_bucket, gate, scale, out_dtype)
+
+
+def gqa_mfma_supported(q, D: int, Dv: int) -> bool:
+    """The matrix-core kernel serves bf16 with head sizes in multiples of
+    32 up to 128; everything else runs the one-wave-per-row kernel."""
+    return (q.dtype == torch.bfloat16 and D % 32 == 0 and Dv % 32 == 0
+            and D <= 128 and Dv <= 128
+            and hasattr(_SEQ_EXT, "seq_gqa_window_attention_mfma"))
+
+
+def moe_route(logits, correction, top: int, groups: int, keep: int):
+    """Router choice for every row of fp32 logits (N, E): s = softmax,
+    choice score = s + correction; experts form ``groups`` equal groups of
+    neighbours, only the ``keep`` groups with the largest best choice score
+    stay eligible; the ``top`` largest eligible choice scores win.  Returns
+    (index int32 (N, top), s at those indices fp32 (N, top))."""
+    if logits.is_cuda:
+        N = logits.shape[0]
+        idx = torch.empty(N, top, dtype=torch.int32, device=logits.device)
+        w = torch.empty(N, top, dtype=torch.float32, device=logits.device)
+        if N:
+            _ext().seq_moe_route(idx, w, logits, correction, groups, keep)
+        return idx, w
+    return R.moe_route(logits, correction, top, groups, keep)
+
+
+def gelu_erf(x):
+    """Exact (erf) GELU; x may be a column slice."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        if x.shape[0]:
+            _ext().seq_act_mul(out, x, x, 3)
+        return out
+    return R.gelu_erf(x)
+
+
+def moe_routed_ffn_supported(h, top: int, ff: int) -> bool:
+    """The fused expert path serves bf16 decode-sized batches on the GPU."""
+    return moe_table_ffn_supported(h, top, ff)
+
+
+def moe_routed_ffn(h, idx, w_up, w_down) -> torch.Tensor:
+    """Router-chosen plain experts: row t*top+k of the result is expert
+    idx[t, k] applied to h[t], W_down gelu_erf(W_up h); rows whose index is
+    >= E (identity experts) are left unwritten.  w_up (E, ff, W), w_down
+    (E, W, ff)."""
+    if h.is_cuda:
+        N, top = idx.shape
+        y = torch.empty(N * top, h.shape[1], dtype=h.dtype, device=h.device)
+        act = torch.empty(N * top, w_down.shape[2], dtype=h.dtype,
+                          device=h.device)
+        _ext().seq_moe_routed_ffn(y, act, h, idx, w_up, w_down)
+        return y
+    return R.moe_routed_ffn(h, idx, w_up, w_down)
+
+
+def moe_weighted_combine(ys, idx, w, h, shared, E: int, weight_eps: float,
+                         out_dtype) -> torch.Tensor:
+    """y[n] = sum_k w'[n,k] * (ys[n*top+k] if idx[n,k] < E else h[n])
+    [+ shared[n]] with w' = w / (sum_k w + weight_eps), fp32 sums."""
+    if ys.is_cuda:
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        if h.shape[0]:
+            _ext().seq_moe_weighted_combine(
+                out, ys, idx, w, h,
+                shared if shared is not None else torch.Tensor(), E,
+                weight_eps)
+        return out
+    return R.moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps,
+                                  out_dtype)
 
 
 def silu_mul_any(gate, up):

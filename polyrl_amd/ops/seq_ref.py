@@ -16,11 +16,11 @@ def _w(weight: torch.Tensor) -> torch.Tensor:
     return weight.float().reshape(-1)
 
 
-def add_rmsnorm_f32res(res, y, weight, eps, out_dtype):
+def add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset=0.0):
     if y is not None:
         res.add_(y.float())
     inv = torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps)
-    return (res * inv * _w(weight)).to(out_dtype)
+    return (res * inv * (_w(weight) + offset)).to(out_dtype)
 
 
 def residual_add_cast(res, y, out_dtype):
@@ -29,10 +29,15 @@ def residual_add_cast(res, y, out_dtype):
     return res if out_dtype == torch.float32 else res.to(out_dtype)
 
 
-def add_scaled_unit_rms(res, y, weight, eps):
+def add_scaled_unit_rms(res, y, weight, eps, offset=0.0):
     yf = y.float()
     inv = torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
-    res.add_(yf * inv * _w(weight))
+    res.add_(yf * inv * (_w(weight) + offset))
+
+
+def add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype, offset):
+    add_scaled_unit_rms(res, y, w_post, eps, offset)
+    return add_rmsnorm_f32res(res, None, w_next, eps, out_dtype, offset)
 
 
 def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,
@@ -213,3 +218,105 @@ def moe_table_ffn(h, tokens, table, w_gu, w_down):
             a = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(h.dtype)
             y[t * top + k] = (w_down[e].float() @ a.float()).to(h.dtype)
     return y
+
+
+def gelu_erf(x):
+    xf = x.float()
+    return (0.5 * xf * (1.0 + torch.erf(xf * (1.0 / math.sqrt(2.0))))
+            ).to(x.dtype)
+
+
+def gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp, positions,
+                      cache, slot_mapping, H, G, D, Dv):
+    N = q.shape[0]
+    qf, kf = q.float(), k.float()
+    vf = kf if v is None else v.float()
+    if q_norm is not None:
+        qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) \
+            * q_norm.float()
+        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) \
+            * k_norm.float()
+    qf, kf = qf.reshape(N, H, D).clone(), kf.reshape(N, G, D).clone()
+    half = 0 if inv_freq is None else inv_freq.numel()
+    if half:
+        ang = positions.float().unsqueeze(-1) * inv_freq.float()
+        c = (torch.cos(ang) * amp).unsqueeze(1)
+        s = (torch.sin(ang) * amp).unsqueeze(1)
+        for t in (qf, kf):
+            a, b = t[..., :half].clone(), t[..., half:2 * half].clone()
+            t[..., :half] = a * c - b * s
+            t[..., half:2 * half] = b * c + a * s
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping.long()] = torch.cat(
+        [kf.reshape(N, G * D), vf.reshape(N, G * Dv)], -1).to(cache.dtype)
+    return qf.reshape(N, H * D).to(q.dtype)
+
+
+def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H, G,
+                         D, Dv, window, keep_first, rel, dist_bucket, gate,
+                         scale, out_dtype):
+    N = q.shape[0]
+    ps = cache.shape[1]
+    flat = cache.view(-1, cache.shape[-1]).float()
+    out = torch.empty(N, H, Dv, dtype=torch.float32, device=q.device)
+    ptab = page_table.tolist()
+    qf = q.float().view(N, H, D)
+    per = H // G
+    for n, (b, p) in enumerate(zip(seq_of_tok.tolist(), positions.tolist())):
+        lo = max(0, p - window + 1)
+        js = list(range(0, min(keep_first, lo))) + list(range(lo, p + 1))
+        rows = torch.tensor([ptab[b][j // ps] * ps + j % ps for j in js],
+                            dtype=torch.long)
+        kv = flat[rows]
+        kk = kv[:, :G * D].view(-1, G, D).repeat_interleave(per, 1)
+        vv = kv[:, G * D:].view(-1, G, Dv).repeat_interleave(per, 1)
+        s = torch.einsum("hd,jhd->hj", qf[n], kk) * scale
+        if rel is not None:
+            dist = torch.tensor([p - j for j in js], dtype=torch.long)
+            s = s + rel.float()[dist_bucket.long()[dist]].t()
+        o = torch.einsum("hj,jhv->hv", torch.softmax(s, -1), vv)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[n].float()).unsqueeze(-1)
+        out[n] = o
+    return out.view(N, H * Dv).to(out_dtype)
+
+
+def moe_route(logits, correction, top, groups, keep):
+    s = torch.softmax(logits.float(), -1)
+    choice = s + correction.float()
+    N, E = s.shape
+    if groups > 1:
+        best = choice.view(N, groups, E // groups).max(-1).values
+        kept = best.topk(keep, -1).indices
+        open_ = torch.zeros(N, groups, dtype=torch.bool, device=s.device)
+        open_.scatter_(1, kept, True)
+        choice = choice.masked_fill(
+            ~open_.repeat_interleave(E // groups, 1), float("-inf"))
+    idx = choice.topk(top, -1).indices
+    return idx.int(), s.gather(1, idx)
+
+
+def moe_routed_ffn(h, idx, w_up, w_down):
+    N, top = idx.shape
+    E = w_up.shape[0]
+    y = torch.zeros(N * top, h.shape[1], dtype=h.dtype, device=h.device)
+    flat = idx.reshape(-1)
+    for e in torch.unique(flat).tolist():
+        if e >= E:
+            continue
+        sl = (flat == e).nonzero().squeeze(1)
+        a = gelu_erf(h[sl // top] @ w_up[e].t())
+        y[sl] = a @ w_down[e].t()
+    return y
+
+
+def moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps, out_dtype):
+    N, top = idx.shape
+    wn = w.float() / (w.float().sum(-1, keepdim=True) + weight_eps)
+    rows = ys.float().view(N, top, -1)
+    ident = (idx >= E).unsqueeze(-1)
+    rows = torch.where(ident, h.float().unsqueeze(1).expand_as(rows), rows)
+    y = (rows * wn.unsqueeze(-1)).sum(1)
+    if shared is not None:
+        y = y + shared.float()
+    return y.to(out_dtype)

@@ -212,6 +212,70 @@ class LatentAttnMixer(_Part):
         return _mm(o, self.wo)
 
 
+class WindowAttnMixer(_Part):
+    """Grouped-query attention over a sliding window of paged K/V rows
+    (models.hybrid.WindowAttnSpec): one fused projection for queries, keys,
+    values (unless the keys serve as values) and the per-head gate; one
+    kernel norms, rotates and writes the cache rows; one attends."""
+
+    def __init__(self, spec, width, device, dtype):
+        self.spec = s = spec
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        f32 = torch.float32
+        self.nq, self.nk = s.heads * s.dim, s.kv_heads * s.dim
+        self.nv = 0 if s.values_from_keys else s.kv_heads * s.vdim
+        self.ng = s.heads if s.head_gate else 0
+        self.row = s.kv_heads * (s.dim + s.vdim)
+        self.w_in = z(self.nq + self.nk + self.nv + self.ng, width)
+        self.q_norm = z(self.nq, dt=f32) if s.qk_norm else None
+        self.k_norm = z(self.nk, dt=f32) if s.qk_norm else None
+        self.wo = z(width, s.heads * s.vdim)
+        self.inv_freq, self.amp = None, 1.0
+        if s.rope is not None:
+            f, self.amp = s.rope.inv_freq_and_amp()
+            self.inv_freq = torch.tensor(f, dtype=torch.float64).float() \
+                .to(device)
+        self.rel = self.dist_bucket = None
+        if s.bias_far > 0:
+            self.rel = z(int(s.bias_rows), s.heads, dt=f32)
+            self.dist_bucket = torch.tensor(
+                s.bucket_of_distance(), dtype=torch.int32).to(device)
+
+    def named(self, p):
+        a, b = self.nq, self.nq + self.nk
+        out = {p + "q": self.w_in[:a], p + "k": self.w_in[a:b],
+               p + "o": self.wo}
+        if self.nv:
+            out[p + "v"] = self.w_in[b:b + self.nv]
+        if self.ng:
+            out[p + "g"] = self.w_in[b + self.nv:]
+        if self.q_norm is not None:
+            out[p + "q.norm"] = self.q_norm
+            out[p + "k.norm"] = self.k_norm
+        if self.rel is not None:
+            out[p + "rel"] = self.rel
+        return out
+
+    def forward(self, h, bt, li, model, cache, states):
+        s = self.spec
+        a, b = self.nq, self.nq + self.nk
+        proj = _mm(h, self.w_in)
+        rows = cache.rows[li]
+        q = seq.gqa_prepare_store(
+            proj.narrow(1, 0, a), proj.narrow(1, a, self.nk),
+            proj.narrow(1, b, self.nv) if self.nv else None,
+            self.q_norm, self.k_norm, model.cfg.norm_eps, self.inv_freq,
+            self.amp, bt.positions, rows, bt.slot_mapping, s.heads,
+            s.kv_heads, s.dim, s.vdim)
+        o = seq.gqa_window_attention(
+            q, rows, bt.page_table, bt.seq_of_tok, bt.positions, s.heads,
+            s.kv_heads, s.dim, s.vdim, s.window, s.keep_first, self.rel,
+            self.dist_bucket,
+            proj.narrow(1, b + self.nv, self.ng) if self.ng else None,
+            s.scale, h.dtype, tiles=bt.attn_tiles)
+        return _mm(o, self.wo)
+
+
 class DenseFF(_Part):
     def __init__(self, spec, width, vocab, device, dtype):
         self.ff = spec.ff
@@ -300,9 +364,76 @@ class TableMoE(_Part):
         return None                       # already in the residual
 
 
+class RoutedMoE(_Part):
+    """Experts chosen by a softmax router (fp32) with a selection-only
+    correction and group-limited choice; plain experts W_down gelu(W_up h);
+    trailing identity experts return the input; a shared expert runs for
+    every token.  Returns the sublayer output (N, width)."""
+
+    def __init__(self, spec, width, vocab, device, dtype):
+        self.spec = f = spec
+        self.E, self.top, self.ff = f.experts, f.top, f.ff
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        f32 = torch.float32
+        self.w_up = z(f.experts, f.ff, width)
+        self.w_down = z(f.experts, width, f.ff)
+        self.router = z(f.experts + f.identity, width, dt=f32)
+        self.correction = z(f.experts + f.identity, dt=f32)
+        self.s_up = z(f.shared_ff, width) if f.shared_ff else None
+        self.s_down = z(width, f.shared_ff) if f.shared_ff else None
+
+    def named(self, p):
+        out = {p + "router": self.router, p + "correction": self.correction}
+        for e in range(self.E):
+            out[f"{p}e{e}.up"] = self.w_up[e]
+            out[f"{p}e{e}.down"] = self.w_down[e]
+        if self.s_up is not None:
+            out[p + "shared.up"] = self.s_up
+            out[p + "shared.down"] = self.s_down
+        return out
+
+    def experts_large(self, h, idx):
+        """Rows sorted by expert, one vendor product pair per live expert
+        (prompt-sized or fp32 batches)."""
+        N, top = idx.shape
+        flat = idx.reshape(-1)
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=self.E + 1)[:self.E].tolist()
+        xs = h.index_select(0, order // top)
+        ys_sorted = torch.empty(N * top, h.shape[1], device=h.device,
+                                dtype=h.dtype)
+        o = 0
+        for e, c in enumerate(counts):
+            if c:
+                act = seq.gelu_erf(_mm(xs[o:o + c], self.w_up[e]))
+                ys_sorted[o:o + c] = _mm(act, self.w_down[e])
+                o += c
+        ys = torch.empty_like(ys_sorted)
+        ys[order] = ys_sorted           # identity rows stay unread
+        return ys
+
+    def forward(self, h, res, bt):
+        f = self.spec
+        logits = _mm(h.float(), self.router)
+        idx, w = seq.moe_route(logits, self.correction, f.top, f.group_count,
+                               f.group_keep)
+        if h.shape[0] <= 256 and self.E and \
+                seq.moe_routed_ffn_supported(h, self.top, self.ff):
+            ys = seq.moe_routed_ffn(h, idx, self.w_up, self.w_down)
+        elif self.E:
+            ys = self.experts_large(h, idx.long())
+        else:
+            ys = h.new_empty(h.shape[0] * f.top, h.shape[1])
+        shared = None
+        if self.s_up is not None:
+            shared = _mm(seq.gelu_erf(_mm(h, self.s_up)), self.s_down)
+        return seq.moe_weighted_combine(ys, idx, w, h, shared, self.E,
+                                        f.weight_eps, h.dtype)
+
+
 _MIXERS = {"general_delta": DeltaRuleMixer, "mamba2": SSMMixer,
-           "latent_attention": LatentAttnMixer}
-_FFS = {"dense": DenseFF, "moe": TableMoE}
+           "latent_attention": LatentAttnMixer, "attention": WindowAttnMixer}
+_FFS = {"dense": DenseFF, "moe": TableMoE, "routed_moe": RoutedMoE}
 
 
 class HybridLayer:
@@ -334,6 +465,31 @@ class HybridLayer:
         return out
 
 
+class SandwichLayer:
+    """x += norm(mixer(norm(x))), x += norm(ff(norm(x))): four per-channel
+    norm weights stored as offsets from ``cfg.norm_offset``."""
+
+    def __init__(self, cfg: HybridConfig, li: int, device, dtype):
+        L = cfg.layers[li]
+        W = cfg.hidden_size
+        z = lambda: torch.empty(W, device=device, dtype=torch.float32)
+        self.norm1, self.norm1b = z(), z()
+        self.mixer = _MIXERS[L.mixer.kind](L.mixer, W, device, dtype)
+        self.ff = None if L.ff is None else \
+            _FFS[L.ff.kind](L.ff, W, cfg.vocab_size, device, dtype)
+        self.norm2, self.norm2b = (z(), z()) if self.ff is not None \
+            else (None, None)
+
+    def named(self, p: str) -> Dict[str, torch.Tensor]:
+        out = {p + "norm1": self.norm1, p + "norm1b": self.norm1b}
+        out.update(self.mixer.named(p + "mix."))
+        if self.ff is not None:
+            out[p + "norm2"] = self.norm2
+            out[p + "norm2b"] = self.norm2b
+            out.update(self.ff.named(p + "mlp."))
+        return out
+
+
 class HybridInferenceModel:
     """Weights + packed forward of a hybrid decoder for the rollout engine
     (same weight-update surface as InferenceModel: ``_name_map``,
@@ -351,14 +507,22 @@ class HybridInferenceModel:
         for L in cfg.layers:                 # sizes the config leaves open
             if L.mixer.kind == "general_delta" and L.mixer.decay_rank is None:
                 L.mixer.decay_rank = max(8, cfg.hidden_size // 12 // 8 * 8)
-        self.layers = [HybridLayer(cfg, li, device, dtype)
+            if L.mixer.kind == "attention" and L.mixer.bias_far > 0 \
+                    and L.mixer.bias_rows is None:
+                raise ValueError("the distance-bias table's rows come from "
+                                 "the checkpoint: call resolve_shapes first")
+        self.sandwich = cfg.layer_style == "sandwich"
+        layer_cls = SandwichLayer if self.sandwich else HybridLayer
+        self.layers = [layer_cls(cfg, li, device, dtype)
                        for li in range(cfg.num_hidden_layers)]
+        self.runs = cfg.run_order()
         W = cfg.hidden_size
         self.embed = torch.empty(cfg.vocab_size, W, device=device, dtype=dtype)
         self.side_embed = torch.empty(
             cfg.vocab_size, cfg.num_hidden_layers * cfg.token_side_dim,
             device=device, dtype=dtype)
-        self.final_norm = torch.empty(1, device=device, dtype=torch.float32)
+        self.final_norm = torch.empty(W if self.sandwich else 1,
+                                      device=device, dtype=torch.float32)
         self.lm_head = torch.empty(cfg.vocab_size, W, device=device,
                                    dtype=dtype)
         self._name_map: Dict[str, torch.Tensor] = {
@@ -380,20 +544,32 @@ class HybridInferenceModel:
                 shp = shapes.get(f"l{li}.mix.w1")
                 if shp is not None:
                     L.mixer.decay_rank = int(shp[0])
+            if L.mixer.kind == "attention" and L.mixer.bias_far > 0:
+                shp = shapes.get(f"l{li}.mix.rel")
+                if shp is not None:
+                    L.mixer.bias_rows = int(shp[0])
         return cfg
 
     def cache_row_dims(self) -> Dict[int, int]:
-        return {li: L.mixer.row for li, L in enumerate(self.layers)
-                if isinstance(L.mixer, LatentAttnMixer) and L.mixer.owner}
+        """Cache row size per layer RUN that owns paged rows (a looped
+        layer owns one set of rows per pass)."""
+        out = {}
+        for ri, li in enumerate(self.runs):
+            m = self.layers[li].mixer
+            if isinstance(m, WindowAttnMixer) or \
+                    (isinstance(m, LatentAttnMixer) and m.owner):
+                out[ri] = m.row
+        return out
 
     def state_shapes(self) -> Dict[tuple, tuple]:
         out = {}
-        for li, L in enumerate(self.layers):
+        for ri, li in enumerate(self.runs):
+            L = self.layers[li]
             if self.cfg.canon_taps > 1:
-                out[(li, "canon")] = (self.cfg.canon_taps - 1,
+                out[(ri, "canon")] = (self.cfg.canon_taps - 1,
                                       self.cfg.hidden_size)
             for k, shp in L.mixer.state_shapes().items():
-                out[(li, k)] = shp
+                out[(ri, k)] = shp
         return out
 
     # ------------------------------------------------------------ weights
@@ -448,6 +624,12 @@ class HybridInferenceModel:
                     torch.rand(buf.shape[0], E, generator=g).argsort(1)[
                         :, :buf.shape[1]].int()
                 buf.copy_(t)
+            elif self.sandwich and name.endswith(
+                    ("norm1", "norm2", "norm1b", "norm2b", "final.norm")):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.1)
+            elif name.endswith(("mix.rel", "mlp.correction")):
+                buf.copy_(torch.randn(buf.shape, generator=g) *
+                          (0.5 if name.endswith("rel") else 0.02))
             elif name.endswith(("norm1", "norm2", "final.norm", ".norm",
                                 "mix.D")):
                 buf.fill_(1.0)
@@ -473,7 +655,7 @@ class HybridInferenceModel:
                 device=states.device)
         return t
 
-    def _moe_of(self, name: str) -> "TableMoE":
+    def _moe_of(self, name: str):
         return self.layers[int(name.split(".")[0][1:])].ff
 
     # ------------------------------------------------------------ forward
@@ -482,6 +664,8 @@ class HybridInferenceModel:
         """Packed rows through every layer; returns the fp32 residual
         stream (N, width) before the final norm.  Writes this step's cache
         rows and advances the sequences' recurrent states in place."""
+        if self.sandwich:
+            return self._forward_sandwich(bt, cache, states)
         cfg, dt = self.cfg, self.dtype
         eps = cfg.norm_eps
         res = self.embed[bt.tokens].float()
@@ -509,12 +693,43 @@ class HybridInferenceModel:
                 self.capture_layers.append(res.clone())
         return res
 
+    def _forward_sandwich(self, bt: HybridBatch, cache, states):
+        """Layer runs of the sandwich style.  Each joint between two
+        sublayers is one fused pass: add the normed sublayer output to the
+        fp32 residual and norm the result for the next sublayer."""
+        cfg, dt = self.cfg, self.dtype
+        eps, off = cfg.norm_eps, cfg.norm_offset
+        res = self.embed[bt.tokens].float()
+        runs = self.runs
+        h = seq.add_rmsnorm_f32res(res, None, self.layers[runs[0]].norm1,
+                                   eps, dt, off) if runs else None
+        for ri, li in enumerate(runs):
+            L = self.layers[li]
+            nxt = self.layers[runs[ri + 1]].norm1 \
+                if ri + 1 < len(runs) else None
+            y = L.mixer.forward(h, bt, ri, self, cache, states)
+            if L.ff is not None:
+                h = seq.add_unit_rms_then_norm(res, y, L.norm1b, L.norm2,
+                                               eps, dt, off)
+                y = L.ff.forward(h, res, bt)
+                post = L.norm2b
+            else:
+                post = L.norm1b
+            if nxt is not None:
+                h = seq.add_unit_rms_then_norm(res, y, post, nxt, eps, dt,
+                                               off)
+            else:
+                seq.add_scaled_unit_rms(res, y, post, eps, off)
+            if self.capture_layers is not None:
+                self.capture_layers.append(res.clone())
+        return res
+
     @torch.no_grad()
     def logits(self, res_rows: torch.Tensor) -> torch.Tensor:
         """Final norm + head on residual rows -> fp32 logits."""
         h = seq.add_rmsnorm_f32res(res_rows.contiguous(), None,
                                    self.final_norm, self.cfg.norm_eps,
-                                   self.dtype)
+                                   self.dtype, self.cfg.norm_offset)
         out = _mm(h, self.lm_head).float()
         if self.cfg.logit_scale != 1.0:
             out = out * self.cfg.logit_scale
