@@ -4,7 +4,8 @@
 #include <torch/extension.h>
 
 void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
-                     torch::Tensor weight, double eps, int64_t mode);
+                     torch::Tensor weight, double eps, int64_t mode,
+                     double offset, torch::Tensor weight2);
 void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                      torch::Tensor bias, torch::Tensor state,
                      torch::Tensor cu_q, torch::Tensor state_slot,
@@ -52,7 +53,42 @@ void seq_latent_attention_mfma(torch::Tensor out, torch::Tensor q,
                                int64_t window, torch::Tensor sink,
                                double scale, int64_t mode);
 
+void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
+                           torch::Tensor k, torch::Tensor v,
+                           torch::Tensor q_norm, torch::Tensor k_norm,
+                           double eps, torch::Tensor inv_freq, double amp,
+                           torch::Tensor positions, torch::Tensor cache,
+                           torch::Tensor slot_mapping, int64_t H, int64_t G,
+                           int64_t D, int64_t Dv);
+void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
+                              torch::Tensor cache, torch::Tensor page_table,
+                              torch::Tensor seq_of_tok,
+                              torch::Tensor positions, int64_t H, int64_t G,
+                              int64_t D, int64_t Dv, int64_t window,
+                              int64_t keep_first, torch::Tensor rel,
+                              torch::Tensor dist_bucket, torch::Tensor gate,
+                              double scale);
+void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
+                   torch::Tensor correction, int64_t groups, int64_t keep);
+void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
+                        torch::Tensor idx, torch::Tensor w_up,
+                        torch::Tensor w_down);
+void seq_moe_weighted_combine(torch::Tensor out, torch::Tensor ys,
+                              torch::Tensor idx, torch::Tensor w,
+                              torch::Tensor h, torch::Tensor shared,
+                              int64_t E, double weight_eps);
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("seq_gqa_prepare_store", &seq_gqa_prepare_store,
+        "whole-row q/k norm + partial rotation + K/V cache rows");
+  m.def("seq_gqa_window_attention", &seq_gqa_window_attention,
+        "grouped-query window attention over paged K/V rows (any dtype)");
+  m.def("seq_moe_route", &seq_moe_route,
+        "softmax router with correction and group-limited top-k");
+  m.def("seq_moe_routed_ffn", &seq_moe_routed_ffn,
+        "router-chosen plain experts for decode-sized bf16 batches");
+  m.def("seq_moe_weighted_combine", &seq_moe_weighted_combine,
+        "weighted sum of chosen experts, identity experts and shared");
   m.def("seq_add_rmsnorm", &seq_add_rmsnorm,
         "fp32 residual add + RMS norm / cast / unit-RMS add");
   m.def("seq_causal_conv", &seq_causal_conv,

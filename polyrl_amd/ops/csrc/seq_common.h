@@ -29,6 +29,10 @@ DEV_INLINE float gelu_tanhf_acc(float z) {
   return 0.5f * z * (1.f + tanhf(c * (z + 0.044715f * z * z * z)));
 }
 
+DEV_INLINE float gelu_erff_acc(float z) {
+  return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+}
+
 // sum over the 2^k lanes l, l^1, ..., l^(G-1) (G a power of two <= 64)
 template <int G>
 DEV_INLINE float lanegroup_sum(float x) {

@@ -13,20 +13,25 @@
 #include "seq_common.h"
 
 // ------------------------------------------------- residual add + RMS norm
-// mode 0: res += y; out = res * rsqrt(mean(res^2)+eps) * w   (w: 1 or D)
-// mode 1: res += y; out = res (cast)                          (no norm)
-// mode 2: res += y * rsqrt(mean(y^2)+eps) * w                 (out unused)
+// g[i] = off + w[i] (w holds 1 or D numbers; off = 0 for plain weights, 1 for
+// weights stored around zero)
+// mode 0: res += y; out = res * rsqrt(mean(res^2)+eps) * g      (norm)
+// mode 1: res += y; out = res (cast)                             (no norm)
+// mode 2: res += y * rsqrt(mean(y^2)+eps) * g                    (out unused)
+// mode 3: mode 2, then out = res * rsqrt(mean(res^2)+eps) * (off + w2)
+//         (the joint between two normed sublayers in one pass)
 template <typename T>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
     T* __restrict__ out, float* __restrict__ res, const T* __restrict__ y,
     long ldy, const float* __restrict__ w, int wn, int D, float eps,
-    int mode, bool out_is_res) {
-  __shared__ float red[8];
+    int mode, bool out_is_res, float off, const float* __restrict__ w2,
+    int w2n) {
+  __shared__ float red[8], red2[8];
   const long row = blockIdx.x;
   float* rr = res + row * D;
   const T* yr = y ? y + row * ldy : nullptr;
   float ss = 0.f;
-  if (mode == 2) {
+  if (mode >= 2) {
     for (int i = threadIdx.x; i < D; i += 256) {
       const float f = ldf(yr + i);
       ss += f * f;
@@ -51,15 +56,25 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
   const float inv = rsqrtf(ss / D + eps);
   if (mode == 0) {
     for (int i = threadIdx.x; i < D; i += 256)
-      stf(out + row * D + i, rr[i] * inv * w[wn == 1 ? 0 : i]);
-  } else {
-    for (int i = threadIdx.x; i < D; i += 256)
-      rr[i] += ldf(yr + i) * inv * w[wn == 1 ? 0 : i];
+      stf(out + row * D + i, rr[i] * inv * (w[wn == 1 ? 0 : i] + off));
+    return;
   }
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < D; i += 256) {
+    const float f = rr[i] + ldf(yr + i) * inv * (w[wn == 1 ? 0 : i] + off);
+    rr[i] = f;
+    ss2 += f * f;
+  }
+  if (mode == 2) return;
+  ss2 = block_reduce_sum<4>(ss2, red2);
+  const float inv2 = rsqrtf(ss2 / D + eps);
+  for (int i = threadIdx.x; i < D; i += 256)   // own writes again
+    stf(out + row * D + i, rr[i] * inv2 * (w2[w2n == 1 ? 0 : i] + off));
 }
 
 void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
-                     torch::Tensor weight, double eps, int64_t mode) {
+                     torch::Tensor weight, double eps, int64_t mode,
+                     double offset, torch::Tensor weight2) {
   CHECK_F32(res);
   TORCH_CHECK(res.dim() == 2);
   const int D = res.size(1);
@@ -70,16 +85,25 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
     CHECK_ROWS(y);
     TORCH_CHECK(y.size(0) == rows && y.size(1) == D, "y shape");
   }
-  TORCH_CHECK(mode != 2 || has_y);
+  TORCH_CHECK(mode >= 0 && mode <= 3);
+  TORCH_CHECK(mode < 2 || has_y);
   const float* w = nullptr;
-  int wn = 0;
+  const float* w2 = nullptr;
+  int wn = 0, w2n = 0;
   if (mode != 1) {
     CHECK_F32(weight);
     wn = weight.numel();
     TORCH_CHECK(wn == 1 || wn == D, "norm weight must hold 1 or D numbers");
     w = weight.data_ptr<float>();
   }
+  if (mode == 3) {
+    CHECK_F32(weight2);
+    w2n = weight2.numel();
+    TORCH_CHECK(w2n == 1 || w2n == D, "norm weight must hold 1 or D numbers");
+    w2 = weight2.data_ptr<float>();
+  }
   const bool out_is_res = out.data_ptr() == res.data_ptr();
+  TORCH_CHECK(mode != 3 || !out_is_res);
   if (mode != 2) {
     TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
                 out.numel() == res.numel());
@@ -93,7 +117,8 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
   SEQ_DISPATCH_T(dt, { hipLaunchKernelGGL((add_rmsnorm_kernel<T>), dim3(rows), dim3(256), 0, stream, 
       mode == 2 || out_is_res ? nullptr : (T*)out.data_ptr(),
       res.data_ptr<float>(), has_y ? (const T*)y.data_ptr() : nullptr,
-      has_y ? y.stride(0) : 0, w, wn, D, (float)eps, (int)mode, out_is_res); });
+      has_y ? y.stride(0) : 0, w, wn, D, (float)eps, (int)mode, out_is_res,
+      (float)offset, w2, w2n); });
   HIP_CHECK_KERNEL();
 }
 
@@ -358,6 +383,7 @@ void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
 
 // ------------------------------------------------------- gated activations
 // mode 0: silu(a) * b   mode 1: sigmoid(a) * b   mode 2: tanh(a)
+// mode 3: gelu(a), the exact (erf) form
 template <typename T>
 __global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
                                long lda, const T* __restrict__ b, long ldb,
@@ -372,6 +398,8 @@ __global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
     float v;
     if (mode == 2) {
       v = tanhf(av);
+    } else if (mode == 3) {
+      v = gelu_erff_acc(av);
     } else {
       const float bv = ldf(b + r * ldb + c);
       v = (mode == 0 ? siluf_acc(av) : sigmoidf_acc(av)) * bv;
