@@ -644,7 +644,7 @@ class Engine:
         if self.hybrid:
             ok = []
             for r in decode_reqs:
-                if self._ensure_pages(1) and \
+                if self._ensure_pages(1, self._seq_ids[r.rid]) and \
                         self.kv.allocate(self._seq_ids[r.rid], 1):
                     ok.append(r)
                 else:
@@ -695,8 +695,18 @@ class Engine:
         return [outs[f"{rid_prefix}-{i}"] for i in range(len(prompts))]
 
     # -------------------------------------------------------------- internals
-    def _ensure_pages(self, num_tokens: int) -> bool:
-        """Free-list check with radix-cache LRU eviction under pressure."""
+    def _ensure_pages(self, num_tokens: int,
+                      seq_id: Optional[int] = None) -> bool:
+        """Free-list check with radix-cache LRU eviction under pressure.
+        With ``seq_id`` the room left in that sequence's last page counts,
+        so a full pool still takes tokens that need no new page."""
+        if seq_id is not None:
+            need = self.kv.pages_needed(seq_id, num_tokens)
+            if need <= self.kv.free_pages:
+                return True
+            if self.radix is not None:
+                self.radix.evict(need - self.kv.free_pages)
+            return need <= self.kv.free_pages
         if self.kv.can_allocate(num_tokens):
             return True
         if self.radix is not None:
@@ -861,7 +871,7 @@ class Engine:
                     self.states.acquire(sid)
                 self._forced[rid] = r
             start = len(r.input_ids)
-            if not self._ensure_pages(len(toks)) or \
+            if not self._ensure_pages(len(toks), self._seq_ids[rid]) or \
                     not self.kv.allocate(self._seq_ids[rid], len(toks)):
                 raise RuntimeError("cache pool exhausted at " + rid)
             r.input_ids.extend(toks)

@@ -52,6 +52,15 @@ class PageAllocator:
     def can_allocate(self, num_tokens: int) -> bool:
         return (num_tokens + self.page_size - 1) // self.page_size <= len(self._free)
 
+    def pages_needed(self, seq_id: Optional[int], num_tokens: int) -> int:
+        """New pages that ``num_tokens`` more tokens of ``seq_id`` take
+        (room left in its last page counts); None = a new sequence."""
+        cur = self._seq_len.get(seq_id, 0) if seq_id is not None else 0
+        have = len(self._seq_pages.get(seq_id, ())) if seq_id is not None \
+            else 0
+        need = (cur + num_tokens + self.page_size - 1) // self.page_size
+        return max(need - have, 0)
+
     def allocate(self, seq_id: int, num_tokens: int) -> bool:
         """Grow seq's allocation to hold num_tokens MORE tokens.  Returns
         False (allocating nothing) if pages are exhausted."""

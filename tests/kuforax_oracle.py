@@ -229,3 +229,52 @@ def forward(cfg, W, tokens, return_layers=False):
     if return_layers:
         return logits, torch.stack(seen)
     return logits
+
+
+def random_weights(cfg, seed=0, bias_rows=8):
+    """name -> tensor for a config; values are bf16-representable so every
+    engine dtype loads them exactly."""
+    g = torch.Generator().manual_seed(seed)
+    Wd, V = int(cfg["width"]), int(cfg["vocab"])
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean) \
+            .bfloat16().float()
+
+    def lin(o, i, gain=1.0):
+        return rnd(o, i, std=gain / math.sqrt(i))
+    W = {"embed": rnd(V, Wd), "final.norm": rnd(Wd, std=0.1),
+         "head": lin(V, Wd)}
+    for li, L in enumerate(cfg["layers"]):
+        p, m = f"l{li}.", L["mixer"]
+        H, G = int(m["heads"]), int(m["kv_heads"])
+        D, Dv = int(m["dim"]), int(m["vdim"])
+        for n in ("norm1", "norm1b"):
+            W[p + n] = rnd(Wd, std=0.1)
+        W[p + "mix.q"], W[p + "mix.k"] = lin(H * D, Wd), lin(G * D, Wd)
+        W[p + "mix.o"] = lin(Wd, H * Dv)
+        if L["type"] == "attention":
+            W[p + "mix.q.norm"] = rnd(H * D, std=0.1, mean=1.0)
+            W[p + "mix.k.norm"] = rnd(G * D, std=0.1, mean=1.0)
+            W[p + "mix.g"] = lin(H, Wd, gain=2.0)
+        else:
+            W[p + "mix.v"] = lin(G * Dv, Wd)
+            W[p + "mix.rel"] = rnd(bias_rows, H)
+        f = L.get("mlp")
+        if f is None:
+            continue
+        for n in ("norm2", "norm2b"):
+            W[p + n] = rnd(Wd, std=0.1)
+        r = f["router"]
+        E, n_id = int(r["experts"]), int(r.get("identity", 0))
+        ff = int(f["expert"]["ff"])
+        for e in range(E):
+            W[f"{p}mlp.e{e}.up"] = lin(ff, Wd)
+            W[f"{p}mlp.e{e}.down"] = lin(Wd, ff)
+        W[p + "mlp.router"] = lin(E + n_id, Wd, gain=3.0)
+        W[p + "mlp.correction"] = rnd(E + n_id, std=0.05)
+        if f.get("shared"):
+            sf = int(f["shared"]["ff"])
+            W[p + "mlp.shared.up"] = lin(sf, Wd)
+            W[p + "mlp.shared.down"] = lin(Wd, sf)
+    return W

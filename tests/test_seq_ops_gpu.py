@@ -267,3 +267,144 @@ def test_latent_attention_matrix_cores(H, R_, rd, window, lens, starts):
         tiles=tiles)
     torch.testing.assert_close(got.cpu().float(), want.float(), rtol=3e-2,
                                atol=3e-2)
+
+
+# --------------------------------- sandwich norms, GQA window attention, router
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("D", [48, 200, 2048])
+def test_offset_norms_and_fused_joint(dt, D):
+    N = 9
+    res, y = rnd(N, D), rnd(N, D + 8, dt=dt)[:, 3:3 + D]
+    wa, wb = rnd(D, scale=0.2), rnd(D, scale=0.2)
+    r0, r1 = res.clone(), res.clone().to(DEV)
+    want = R.add_unit_rms_then_norm(r0, y, wa, wb, 1e-5, dt, 1.0)
+    got = seq.add_unit_rms_then_norm(r1, y.to(DEV), wa.to(DEV), wb.to(DEV),
+                                     1e-5, dt, 1.0)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+    seq.add_scaled_unit_rms(r1, y.to(DEV), wb.to(DEV), 1e-5, 1.0)
+    R.add_scaled_unit_rms(r0, y, wb, 1e-5, 1.0)
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+    got = seq.add_rmsnorm_f32res(r1, None, wa.to(DEV), 1e-5, dt, 1.0)
+    want = R.add_rmsnorm_f32res(r0, None, wa, 1e-5, dt, 1.0)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+def _paged(lens, starts, page, row, dt):
+    """Page tables for sequences of starts[b]+lens[b] tokens on shuffled
+    pages, and the packed batch of each one's last lens[b] tokens."""
+    total = [s + n for s, n in zip(starts, lens)]
+    need = [-(-t // page) for t in total]
+    perm = torch.randperm(sum(need) + 3).tolist()
+    ptab = torch.zeros(len(lens), max(need), dtype=torch.int32)
+    o = 0
+    for b, k in enumerate(need):
+        ptab[b, :k] = torch.tensor(perm[o:o + k], dtype=torch.int32)
+        o += k
+    cache = rnd(sum(need) + 3, page, row, dt=dt)
+    pos, sot, slot = [], [], []
+    for b, (s, n) in enumerate(zip(starts, lens)):
+        for p in range(s, s + n):
+            pos.append(p)
+            sot.append(b)
+            slot.append(int(ptab[b, p // page]) * page + p % page)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    return cache, ptab, i32(pos), i32(sot), i32(slot)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv,half,norm,own_v", [
+    (4, 2, 24, 24, 4, True, False), (6, 3, 64, 64, 32, True, False),
+    (4, 1, 16, 40, 0, False, True), (2, 2, 128, 128, 16, True, False),
+    (8, 2, 32, 32, 8, False, True)])
+def test_gqa_prepare_store(dt, H, G, D, Dv, half, norm, own_v):
+    lens, starts, page = [5, 1, 3], [0, 37, 6], 4
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, G * (D + Dv), dt)
+    N = sum(lens)
+    big = rnd(N, H * D + G * D + G * Dv + 5, dt=dt)
+    q, k = big[:, :H * D], big[:, H * D:H * D + G * D]
+    v = big[:, H * D + G * D:H * D + G * D + G * Dv] if own_v else None
+    qn = (rnd(H * D, scale=0.2) + 1) if norm else None
+    kn = (rnd(G * D, scale=0.2) + 1) if norm else None
+    inv = torch.rand(half) if half else None
+    c0, c1 = cache.clone(), cache.clone().to(DEV)
+    want = R.gqa_prepare_store(q, k, v, qn, kn, 1e-5, inv, 1.07, pos, c0, slot,
+                               H, G, D, Dv)
+    g = lambda t: None if t is None else t.to(DEV)
+    got = seq.gqa_prepare_store(g(big)[:, :H * D],
+                                g(big)[:, H * D:H * D + G * D],
+                                None if v is None else
+                                g(big)[:, H * D + G * D:H * D + G * D + G * Dv],
+                                g(qn), g(kn), 1e-5, g(inv), 1.07, g(pos), c1,
+                                g(slot), H, G, D, Dv)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(c1.cpu().float(), c0.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv,window,keep,bias,gate,lens,starts", [
+    (4, 2, 24, 24, 7, 2, False, True, [5, 1, 3], [0, 37, 6]),
+    (6, 3, 64, 64, 16, 5, False, True, [40, 1, 1, 2], [3, 70, 0, 15]),
+    (4, 1, 16, 40, 9, 0, True, False, [5, 1, 30], [0, 37, 6]),
+    (2, 2, 128, 128, 33, 4, False, False, [70, 1], [10, 200]),
+    (8, 2, 32, 96, 20, 0, True, False, [64, 1, 9], [0, 19, 64]),
+    (3, 3, 200, 72, 5, 1, False, True, [6, 2], [0, 9]),
+])
+def test_gqa_window_attention(dt, H, G, D, Dv, window, keep, bias, gate,
+                              lens, starts):
+    page = 4
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, G * (D + Dv), dt)
+    cache = (cache.float() * 0.5).to(dt)
+    N = sum(lens)
+    q = rnd(N, H * D, dt=dt)
+    rel = rnd(10, H) if bias else None
+    dist = torch.randint(0, 10, (window,), dtype=torch.int32) if bias else None
+    gfull = rnd(N, H + 3, dt=dt)
+    gt = gfull[:, 1:1 + H] if gate else None
+    gfull = gfull.to(DEV)
+    scale = 1.0 / math.sqrt(D)
+    want = R.gqa_window_attention(q, cache, ptab, sot, pos, H, G, D, Dv,
+                                  window, keep, rel, dist, gt, scale, dt)
+    g = lambda t: None if t is None else t.to(DEV)
+    tiles = seq.attention_tiles(lens, DEV)
+    for tl in (None, tiles):                 # one wave per row; matrix cores
+        got = seq.gqa_window_attention(
+            g(q), g(cache), g(ptab), g(sot), g(pos), H, G, D, Dv, window,
+            keep, g(rel), g(dist),
+            None if gt is None else gfull[:, 1:1 + H], scale, dt, tiles=tl)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("N,top,E,n_id", [(1, 2, 4, 1), (37, 3, 5, 2),
+                                          (64, 1, 2, 0), (200, 2, 6, 2)])
+def test_routed_experts_bf16(N, top, E, n_id):
+    dt = torch.bfloat16
+    Wd, ff = 96, 64
+    h = rnd(N, Wd, dt=dt)
+    idx = torch.stack([torch.randperm(E + n_id)[:top] for _ in range(N)]).int()
+    w = torch.rand(N, top)
+    up, down = rnd(E, ff, Wd, dt=dt, scale=0.1), rnd(E, Wd, ff, dt=dt, scale=0.1)
+    shared = rnd(N, Wd, dt=dt)
+    ys0 = R.moe_routed_ffn(h, idx, up, down)
+    want = R.moe_weighted_combine(ys0, idx, w, h, shared, E, 1e-20, dt)
+    assert seq.moe_routed_ffn_supported(h.to(DEV), top, ff)
+    ys1 = seq.moe_routed_ffn(h.to(DEV), idx.to(DEV), up.to(DEV), down.to(DEV))
+    real = (idx < E).reshape(-1)
+    torch.testing.assert_close(ys1.cpu().float()[real], ys0.float()[real],
+                               **tol(dt))
+    got = seq.moe_weighted_combine(ys1, idx.to(DEV), w.to(DEV), h.to(DEV),
+                                   shared.to(DEV), E, 1e-20, dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    got = seq.moe_weighted_combine(ys1.float(), idx.to(DEV), w.to(DEV),
+                                   h.to(DEV).float(), None, E, 1e-20,
+                                   torch.float32)
+    want = R.moe_weighted_combine(ys0.float(), idx, w, h.float(), None, E,
+                                  1e-20, torch.float32)
+    torch.testing.assert_close(got.cpu()[:, :], want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_gelu_erf(dt):
+    x = rnd(33, 70, dt=dt, scale=2.0)
+    torch.testing.assert_close(seq.gelu_erf(x.to(DEV)[:, 3:60]).cpu().float(),
+                               R.gelu_erf(x[:, 3:60]).float(), **tol(dt))
