@@ -354,9 +354,10 @@ def test_gqa_window_attention(dt, H, G, D, Dv, window, keep, bias, gate,
                               lens, starts):
     page = 4
     cache, ptab, pos, sot, slot = _paged(lens, starts, page, G * (D + Dv), dt)
-    cache = (cache.float() * 0.5).to(dt)
     N = sum(lens)
-    q = rnd(N, H * D, dt=dt)
+    # peaky softmax (score spread of several units): one key missing or one
+    # too many moves the output far beyond the tolerance
+    q = rnd(N, H * D, dt=dt, scale=2.5)
     rel = rnd(10, H) if bias else None
     dist = torch.randint(0, 10, (window,), dtype=torch.int32) if bias else None
     gfull = rnd(N, H + 3, dt=dt)
