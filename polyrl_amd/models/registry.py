@@ -88,6 +88,16 @@ MODEL_CONFIGS = {
         arch="llama", vocab_size=128256, hidden_size=8192, intermediate_size=28672,
         num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8,
         max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5),
+    # engine-compare partners of the hybrid presets: a 0.4B-class stack and
+    # 8 layers of the 8B layer sizes
+    "llama-400m": DecoderConfig(
+        arch="llama", vocab_size=32000, hidden_size=1024, intermediate_size=4096,
+        num_hidden_layers=12, num_attention_heads=16, num_key_value_heads=4,
+        head_dim=64, max_position_embeddings=8192, rope_theta=500000.0),
+    "llama3-8b-l8": DecoderConfig(
+        arch="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+        num_hidden_layers=8, num_attention_heads=32, num_key_value_heads=8,
+        max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5),
     # 1B-class model for single-GPU sanity benches
     "llama3-1b": DecoderConfig(
         arch="llama", vocab_size=128256, hidden_size=2048, intermediate_size=8192,
@@ -104,7 +114,15 @@ def _hybrid_presets():
             width=64, layers=3, vocab=300, heads=4, kv_heads=2, experts=6,
             top=2, identity=2, expert_ff=32, shared_ff=48, window=24,
             keep_first=3, bias_every=3, loop=(1, 3, 2)),
-        # layer sizes of a ~1B-class model (bench: beside llama3-1b)
+        # bench pairs: beside llama-400m / llama3-1b / llama3-8b-l8
+        "kuforax-400m": lambda: kuforax_preset(
+            width=1024, layers=12, vocab=32000, heads=16, kv_heads=4,
+            experts=8, top=2, identity=2, expert_ff=2048, shared_ff=2048,
+            window=512, keep_first=4),
+        "kuforax-8b-l8": lambda: kuforax_preset(
+            width=4096, layers=8, vocab=128256, heads=32, kv_heads=8,
+            experts=16, top=2, identity=2, expert_ff=3584, shared_ff=7168,
+            window=2048, keep_first=4),
         "kuforax-1b": lambda: kuforax_preset(
             width=2048, layers=16, vocab=128256, heads=32, kv_heads=8,
             experts=16, top=2, identity=2, expert_ff=2560, shared_ff=2560,

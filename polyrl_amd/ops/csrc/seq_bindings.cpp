@@ -68,6 +68,13 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
                               double scale);
+void seq_gqa_window_attention_mfma(
+    torch::Tensor out, torch::Tensor q, torch::Tensor tile_n0,
+    torch::Tensor tile_cnt, torch::Tensor cache, torch::Tensor page_table,
+    torch::Tensor seq_of_tok, torch::Tensor positions, int64_t H, int64_t G,
+    int64_t D, int64_t Dv, int64_t window, int64_t keep_first,
+    torch::Tensor rel, torch::Tensor dist_bucket, torch::Tensor gate,
+    double scale);
 void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
                    torch::Tensor correction, int64_t groups, int64_t keep);
 void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
@@ -83,6 +90,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "whole-row q/k norm + partial rotation + K/V cache rows");
   m.def("seq_gqa_window_attention", &seq_gqa_window_attention,
         "grouped-query window attention over paged K/V rows (any dtype)");
+  m.def("seq_gqa_window_attention_mfma", &seq_gqa_window_attention_mfma,
+        "grouped-query window attention on the matrix cores (bf16)");
   m.def("seq_moe_route", &seq_moe_route,
         "softmax router with correction and group-limited top-k");
   m.def("seq_moe_routed_ffn", &seq_moe_routed_ffn,

@@ -284,7 +284,8 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
                     window, keep_first, rel if rel is not None else e,
                     dist_bucket if dist_bucket is not None else e,
                     gate if gate is not None else e, scale)
-            if tiles is not None and gqa_mfma_supported(q, D, Dv):
+            if tiles is not None and tiles[2] == 0 and \
+                    gqa_mfma_supported(q, D, Dv):
                 _ext().seq_gqa_window_attention_mfma(out, q, tiles[0],
                                                      tiles[1], *args)
             else:
@@ -296,11 +297,11 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
 
 
 def gqa_mfma_supported(q, D: int, Dv: int) -> bool:
-    """The matrix-core kernel serves bf16 with head sizes in multiples of
-    32 up to 128; everything else runs the one-wave-per-row kernel."""
-    return (q.dtype == torch.bfloat16 and D % 32 == 0 and Dv % 32 == 0
-            and D <= 128 and Dv <= 128
-            and hasattr(_SEQ_EXT, "seq_gqa_window_attention_mfma"))
+    """The matrix-core kernel serves bf16 batches that hold a prompt
+    portion, with head sizes in multiples of 8 up to 128; everything else
+    (fp32, odd sizes, steps of single tokens) runs one wave per row."""
+    return (q.dtype == torch.bfloat16 and D % 8 == 0 and Dv % 8 == 0
+            and D <= 128 and Dv <= 128)
 
 
 def moe_route(logits, correction, top: int, groups: int, keep: int):
