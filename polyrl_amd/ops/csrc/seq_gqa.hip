@@ -11,12 +11,12 @@
 // and sin scaled by ``amp``; keys go to the cache row, queries to q_out;
 // values are a separate projection or the key projection as it came in.
 //
-// gqa_attn_kernel: one wave per (token, head), the exactness path (fp32
-// activations, odd head sizes).  A row at position p sees key j <= p when
-// p - j < window or j < keep; the two key ranges [0, min(keep, lo)) and
-// [lo, p] are walked as one list.  Scores, the optional distance-bucket bias
-// rel[bucket[p-j], head], the online softmax and the per-head sigmoid gate
-// are fp32.
+// gqa_attn_kernel: one wave per (token, head): decode steps in either type,
+// and the exactness path (fp32 activations, odd head sizes).  A row at
+// position p sees key j <= p when p - j < window or j < keep; the two key
+// ranges [0, min(keep, lo)) and [lo, p] are walked as one list.  Scores, the
+// optional distance-bucket bias rel[bucket[p-j], head], the online softmax
+// and the per-head sigmoid gate are fp32.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -131,8 +131,51 @@ void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
   HIP_CHECK_KERNEL();
 }
 
-template <typename T, int NCH, int KB>
-__global__ __launch_bounds__(64) void gqa_attn_kernel(
+// dot(q_s[0..D), row[0..D)) with 16-byte loads when the rows allow them
+template <typename T>
+DEV_INLINE float dot_row(const T* __restrict__ r, const float* __restrict__ qs,
+                         int D, bool vec);
+template <>
+DEV_INLINE float dot_row<bf16_t>(const bf16_t* __restrict__ r,
+                                 const float* __restrict__ qs, int D,
+                                 bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int d = 0; d < D; d += 8) {
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(r + d);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc += bf2f(v.v[k]) * qs[d + k];
+    }
+  } else {
+    for (int d = 0; d < D; ++d) acc += bf2f(r[d]) * qs[d];
+  }
+  return acc;
+}
+template <>
+DEV_INLINE float dot_row<float>(const float* __restrict__ r,
+                                const float* __restrict__ qs, int D,
+                                bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int d = 0; d < D; d += 4) {
+      const f32x4v v = *reinterpret_cast<const f32x4v*>(r + d);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc += v.v[k] * qs[d + k];
+    }
+  } else {
+    for (int d = 0; d < D; ++d) acc += r[d] * qs[d];
+  }
+  return acc;
+}
+
+// One wave per (token, head), four heads of a token per block (they share
+// their key/value group's rows in cache when H/G >= 4).  Keys are walked 64
+// at a time in two phases: lane = key for the scores (each lane reads its
+// key row against the query in LDS), then lane = value entry for the
+// weighted sum (the wave reads one value row per key, coalesced, weights
+// and row numbers from LDS).  The waves never meet at a block barrier.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void gqa_attn_kernel(
     T* __restrict__ out,                // (N, H*Dv)
     const T* __restrict__ q,            // (N, H*D) contiguous
     const T* __restrict__ cache,        // (pages*page_size, G*(D+Dv))
@@ -142,10 +185,14 @@ __global__ __launch_bounds__(64) void gqa_attn_kernel(
     const int* __restrict__ dist_bucket,   // (window,) or null
     const T* __restrict__ gate, long ldg,  // (N, H) view or null
     int H, int G, int D, int Dv, int page_size, int window, int keep,
-    float scale) {
+    float scale, bool vec) {
+  __shared__ float q_sh[4][NCH * 64];
+  __shared__ float p_sh[4][64];
+  __shared__ int slot_sh[4][64];
   const long n = blockIdx.x;
-  const int h = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * 4 + wid;
+  if (h >= H) return;                   // whole wave
   const int g = h / (H / G);
   const int row = G * (D + Dv);
   const int koff = g * D, voff = G * D + g * Dv;
@@ -155,63 +202,44 @@ __global__ __launch_bounds__(64) void gqa_attn_kernel(
   const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int nkeep = keep < lo ? keep : lo;
   const int total = nkeep + (pos - lo + 1);
+  float* qs = q_sh[wid];
+  float* ps = p_sh[wid];
+  int* ss = slot_sh[wid];
+  for (int d = lane; d < D; d += 64) qs[d] = ldf(q + (n * H + h) * D + d);
 
-  float qv[NCH], o[NCH];
+  float o[NCH];
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    const int d = lane + 64 * c;
-    qv[c] = d < D ? ldf(q + (n * H + h) * D + d) : 0.f;
-    o[c] = 0.f;
-  }
+  for (int c = 0; c < NCH; ++c) o[c] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  for (int i0 = 0; i0 < total; i0 += KB) {
-    float vv[KB][NCH], s[KB];
-    int jj[KB];
+  for (int base = 0; base < total; base += 64) {
+    const int i = base + lane;
+    const bool valid = i < total;
+    const int ii = valid ? i : total - 1;
+    const int j = ii < nkeep ? ii : lo + (ii - nkeep);
+    const int slot = ptab[j / page_size] * page_size + j % page_size;
+    float s = dot_row<T>(cache + (long)slot * row + koff, qs, D, vec) * scale;
+    if (rel) s += rel[(long)dist_bucket[pos - j] * H + h];
+    if (!valid) s = -INFINITY;
+    const float mn = fmaxf(m, wave_reduce_max(s));
+    const float p = valid ? expf(s - mn) : 0.f;
+    const float corr = expf(m - mn);
+    l = l * corr + wave_reduce_sum(p);
+    m = mn;
+    ps[lane] = p;
+    ss[lane] = slot;
+    const int cntk = total - base < 64 ? total - base : 64;
 #pragma unroll
-    for (int t = 0; t < KB; ++t) {
-      const int i = i0 + t < total ? i0 + t : total - 1;
-      const int j = i < nkeep ? i : lo + (i - nkeep);
-      jj[t] = j;
-      const long r0 = ((long)ptab[j / page_size] * page_size + j % page_size) * row;
-      float acc = 0.f;
+    for (int c = 0; c < NCH; ++c) o[c] *= corr;
+#pragma unroll 4
+    for (int jj = 0; jj < cntk; ++jj) {
+      const float pj = ps[jj];
+      const T* vr = cache + (long)ss[jj] * row + voff;
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int d = lane + 64 * c;
-        const float kvv = d < D ? ldf(cache + r0 + koff + d) : 0.f;
-        vv[t][c] = d < Dv ? ldf(cache + r0 + voff + d) : 0.f;
-        acc += qv[c] * kvv;
+        if (d < Dv) o[c] += pj * ldf(vr + d);
       }
-      s[t] = acc;
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-#pragma unroll
-      for (int t = 0; t < KB; ++t) s[t] += __shfl_xor(s[t], off, WAVE_SIZE);
-    }
-    float mn = m;
-#pragma unroll
-    for (int t = 0; t < KB; ++t) {
-      s[t] *= scale;
-      if (rel) s[t] += rel[(long)dist_bucket[pos - jj[t]] * H + h];
-      if (i0 + t < total) mn = fmaxf(mn, s[t]);
-    }
-    const float corr = expf(m - mn);
-    float p[KB];
-    float ls = 0.f;
-#pragma unroll
-    for (int t = 0; t < KB; ++t) {
-      p[t] = (i0 + t < total) ? expf(s[t] - mn) : 0.f;
-      ls += p[t];
-    }
-    l = l * corr + ls;
-    m = mn;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      float acc = o[c] * corr;
-#pragma unroll
-      for (int t = 0; t < KB; ++t) acc += p[t] * vv[t][c];
-      o[c] = acc;
     }
   }
   float inv = 1.f / l;
@@ -261,15 +289,15 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
 }
 
 #define GQA_LAUNCH(NCHV)                                                      \
-  hipLaunchKernelGGL((gqa_attn_kernel<T, NCHV, 4>), dim3(N, H), dim3(64), 0,  \
-      stream, (T*)out.data_ptr(), (const T*)q.data_ptr(),                     \
+  hipLaunchKernelGGL((gqa_attn_kernel<T, NCHV>), dim3(N, (H + 3) / 4),       \
+      dim3(256), 0, stream, (T*)out.data_ptr(), (const T*)q.data_ptr(),                     \
       (const T*)cache.data_ptr(), page_table.data_ptr<int>(),                 \
       (int)page_table.size(1), seq_of_tok.data_ptr<int>(),                    \
       positions.data_ptr<int>(), has_rel ? rel.data_ptr<float>() : nullptr,   \
       has_rel ? dist_bucket.data_ptr<int>() : nullptr,                        \
       has_gate ? (const T*)gate.data_ptr() : nullptr,                         \
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
-      (int)cache.size(1), (int)window, (int)keep_first, (float)scale)
+      (int)cache.size(1), (int)window, (int)keep_first, (float)scale, vec)
 
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
@@ -287,6 +315,9 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
   const bool has_gate = gate.defined() && gate.numel() > 0;
   const int nch = (int)((std::max(D, Dv) + 63) / 64);
   TORCH_CHECK(nch <= 8, "head sizes above 512 are not supported");
+  // 16-byte row loads need every head's keys to start on a 16-byte border
+  const int per16 = q.scalar_type() == torch::kBFloat16 ? 8 : 4;
+  const bool vec = D % per16 == 0 && Dv % per16 == 0;
   auto stream = at::hip::getCurrentHIPStream();
   SEQ_DISPATCH_T(q.scalar_type(), {
     switch (nch) {
