@@ -1,8 +1,10 @@
 """Configuration of hybrid decoders: a stack whose layers each pick one
-sequence mixer (recurrent, state-space or windowed latent attention) and one
-feed-forward (dense, table-routed experts, or none).
+sequence mixer (recurrent, state-space, windowed latent attention or
+grouped-query window attention) and one feed-forward (dense, table-routed
+experts, router-chosen experts, or none).
 
-The Bizusun design is the first family described this way.  Everything that
+The Bizusun design is the first family described this way, Kuforax the
+second.  Everything that
 can differ between two models of a family is a field here and is read from
 the checkpoint's ``config.json``; constants that the design fixes (the decay
 constant of the delta rule, its key epsilon) are defaults of the mixer

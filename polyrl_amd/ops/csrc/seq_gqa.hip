@@ -141,6 +141,7 @@ DEV_INLINE float dot_row<bf16_t>(const bf16_t* __restrict__ r,
                                  bool vec) {
   float acc = 0.f;
   if (vec) {
+#pragma unroll 4
     for (int d = 0; d < D; d += 8) {
       const bf16x8 v = *reinterpret_cast<const bf16x8*>(r + d);
 #pragma unroll
@@ -157,6 +158,7 @@ DEV_INLINE float dot_row<float>(const float* __restrict__ r,
                                 bool vec) {
   float acc = 0.f;
   if (vec) {
+#pragma unroll 4
     for (int d = 0; d < D; d += 4) {
       const f32x4v v = *reinterpret_cast<const f32x4v*>(r + d);
 #pragma unroll
@@ -168,12 +170,37 @@ DEV_INLINE float dot_row<float>(const float* __restrict__ r,
   return acc;
 }
 
+// 16 bytes of a value row as floats
+template <typename T>
+struct Vec16;
+template <>
+struct Vec16<bf16_t> {
+  static constexpr int N = 8;
+  static DEV_INLINE void load(const bf16_t* p, float* o) {
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = bf2f(v.v[k]);
+  }
+};
+template <>
+struct Vec16<float> {
+  static constexpr int N = 4;
+  static DEV_INLINE void load(const float* p, float* o) {
+    const f32x4v v = *reinterpret_cast<const f32x4v*>(p);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = v.v[k];
+  }
+};
+
 // One wave per (token, head), four heads of a token per block (they share
 // their key/value group's rows in cache when H/G >= 4).  Keys are walked 64
 // at a time in two phases: lane = key for the scores (each lane reads its
 // key row against the query in LDS), then lane = value entry for the
-// weighted sum (the wave reads one value row per key, coalesced, weights
-// and row numbers from LDS).  The waves never meet at a block barrier.
+// weighted sum (weights and row numbers from LDS).  When a value row is
+// ``lpr`` 16-byte pieces with lpr a power of two, lpr lanes read one row and
+// the wave reads 64/lpr rows per load; the lane groups' partial sums meet in
+// a shuffle reduction at the end.  Otherwise (lpr = 0) the wave reads one
+// value row per key.  The waves never meet at a block barrier.
 template <typename T, int NCH>
 __global__ __launch_bounds__(256) void gqa_attn_kernel(
     T* __restrict__ out,                // (N, H*Dv)
@@ -185,7 +212,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
     const int* __restrict__ dist_bucket,   // (window,) or null
     const T* __restrict__ gate, long ldg,  // (N, H) view or null
     int H, int G, int D, int Dv, int page_size, int window, int keep,
-    float scale, bool vec) {
+    float scale, bool vec, int lpr) {
+  constexpr int EPL = Vec16<T>::N;
   __shared__ float q_sh[4][NCH * 64];
   __shared__ float p_sh[4][64];
   __shared__ int slot_sh[4][64];
@@ -207,10 +235,15 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
   int* ss = slot_sh[wid];
   for (int d = lane; d < D; d += 64) qs[d] = ldf(q + (n * H + h) * D + d);
 
-  float o[NCH];
+  float o[NCH], ov[EPL];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) o[c] = 0.f;
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) ov[k] = 0.f;
   float m = -INFINITY, l = 0.f;
+  const int kgrp = lpr ? lane / lpr : 0;          // key of an iteration
+  const int dcol = lpr ? (lane % lpr) * EPL : 0;  // first value entry
+  const int kper = lpr ? 64 / lpr : 1;            // keys per iteration
 
   for (int base = 0; base < total; base += 64) {
     const int i = base + lane;
@@ -229,6 +262,22 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
     ps[lane] = p;
     ss[lane] = slot;
     const int cntk = total - base < 64 ? total - base : 64;
+    if (lpr) {
+#pragma unroll
+      for (int k = 0; k < EPL; ++k) ov[k] *= corr;
+#pragma unroll 4
+      for (int jj0 = 0; jj0 < cntk; jj0 += kper) {
+        const int jj = jj0 + kgrp;
+        if (jj < cntk) {
+          const float pj = ps[jj];
+          float vv[EPL];
+          Vec16<T>::load(cache + (long)ss[jj] * row + voff + dcol, vv);
+#pragma unroll
+          for (int k = 0; k < EPL; ++k) ov[k] += pj * vv[k];
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) o[c] *= corr;
 #pragma unroll 4
@@ -244,6 +293,18 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
   }
   float inv = 1.f / l;
   if (gate) inv *= sigmoidf_acc(ldf(gate + n * ldg + h));
+  if (lpr) {
+#pragma unroll
+    for (int k = 0; k < EPL; ++k)
+      for (int off = lpr; off < 64; off <<= 1)
+        ov[k] += __shfl_xor(ov[k], off, WAVE_SIZE);
+    if (lane < lpr) {
+#pragma unroll
+      for (int k = 0; k < EPL; ++k)
+        stf(out + (n * H + h) * Dv + dcol + k, ov[k] * inv);
+    }
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int d = lane + 64 * c;
@@ -297,7 +358,8 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
       has_rel ? dist_bucket.data_ptr<int>() : nullptr,                        \
       has_gate ? (const T*)gate.data_ptr() : nullptr,                         \
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
-      (int)cache.size(1), (int)window, (int)keep_first, (float)scale, vec)
+      (int)cache.size(1), (int)window, (int)keep_first, (float)scale, vec,     \
+      lpr)
 
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
@@ -318,6 +380,9 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
   // 16-byte row loads need every head's keys to start on a 16-byte border
   const int per16 = q.scalar_type() == torch::kBFloat16 ? 8 : 4;
   const bool vec = D % per16 == 0 && Dv % per16 == 0;
+  // lanes per value row of 16-byte pieces, when that is a power of two <= 64
+  int lpr = vec ? (int)(Dv / per16) : 0;
+  if (lpr > 64 || (lpr & (lpr - 1))) lpr = 0;
   auto stream = at::hip::getCurrentHIPStream();
   SEQ_DISPATCH_T(q.scalar_type(), {
     switch (nch) {

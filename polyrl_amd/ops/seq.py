@@ -1,6 +1,8 @@
-"""Sequence-mixer ops for hybrid decoders: fp32-residual norms, stateful
-causal convolutions, the generalised delta rule, the selective state-space
-scan, and windowed latent attention with a softmax sink.
+"""Sequence-mixer ops for hybrid decoders: fp32-residual norms (plain and
+offset weights, fused joints), stateful causal convolutions, the generalised
+delta rule, the selective state-space scan, windowed latent attention with a
+softmax sink, grouped-query window attention over paged K/V rows, and
+table-routed or router-chosen expert feed-forwards.
 
 Same policy as the rest of ``polyrl_amd.ops``: on a HIP device the in-tree
 extension is REQUIRED (csrc/seq_*.hip, templated on the activation type:

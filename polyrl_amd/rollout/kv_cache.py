@@ -202,10 +202,13 @@ class PagedKVCache(PageAllocator):
 
 
 class PagedLatentCache(PageAllocator):
-    """One row per token and owning layer: ``rows[li]`` is
-    (num_pages, page_size, row_dim[li]) for every layer li that writes a
-    latent cache (normed latent followed by the rotated shared key part).
-    Layers that read another layer's cache hold no tensor of their own."""
+    """One row per token and owning layer run: ``rows[i]`` is
+    (num_pages, page_size, row_dim[i]) for every layer run i that writes
+    cache rows: a normed latent followed by the rotated shared key part
+    (latent attention), or all key heads followed by all value heads
+    (grouped-query window attention).  Layers that read another layer's
+    cache hold no tensor of their own; a looped layer owns one entry per
+    pass."""
 
     def __init__(self, row_dims: Dict[int, int], num_pages: int,
                  page_size: int = 16, dtype: torch.dtype = torch.bfloat16,
