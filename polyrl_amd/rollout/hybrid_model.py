@@ -393,11 +393,12 @@ class RoutedMoE(_Part):
         return out
 
     def experts_large(self, h, idx):
-        """Rows sorted by expert, one vendor product pair per live expert
-        (prompt-sized or fp32 batches)."""
+        """Rows sorted by expert on the device, one vendor product pair per
+        live expert (prompt-sized or fp32 batches); one host sync for the
+        row counts."""
         N, top = idx.shape
         flat = idx.reshape(-1)
-        order = torch.argsort(flat, stable=True)
+        order = torch.argsort(flat, stable=True)     # identity slots last
         counts = torch.bincount(flat, minlength=self.E + 1)[:self.E].tolist()
         xs = h.index_select(0, order // top)
         ys_sorted = torch.empty(N * top, h.shape[1], device=h.device,

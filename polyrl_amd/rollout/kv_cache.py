@@ -160,12 +160,10 @@ class PageAllocator:
     # --------------------------------------------------------------- indexing
     def slots_for(self, seq_id: int, start: int, count: int) -> torch.Tensor:
         """slot ids (page*page_size + off) for token positions [start, start+count)."""
-        pages = self._seq_pages[seq_id]
-        out = torch.empty(count, dtype=torch.int32)
-        for i in range(count):
-            pos = start + i
-            out[i] = pages[pos // self.page_size] * self.page_size + pos % self.page_size
-        return out
+        pages = torch.tensor(self._seq_pages[seq_id], dtype=torch.int64)
+        pos = torch.arange(start, start + count, dtype=torch.int64)
+        return (pages[pos // self.page_size] * self.page_size
+                + pos % self.page_size).to(torch.int32)
 
     def page_table(self, seq_ids: List[int], max_pages: Optional[int] = None
                    ) -> torch.Tensor:

@@ -217,6 +217,23 @@ def test_router_kernel_matches_oracle():
 
 
 @pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("skewed", [False, True])
+def test_prompt_sized_expert_batches(target, skewed):
+    """300 rows take the sorted per-expert products, with routing spread
+    over the experts and with every token sent to one of them."""
+    cfg = config([(bias_attn(window=5), moe(experts=8, top=1, identity=0,
+                                            groups=1, keep=1, shared=0))])
+    W = O.random_weights(cfg, seed=9)
+    if skewed:
+        W["l0.mlp.correction"].zero_()
+        W["l0.mlp.correction"][3] = 4.0
+    t = toks(300, seed=8)
+    e = engine(cfg, W, target, tokens=320)
+    want = O.forward(cfg, W, t)
+    close(run(e, "a", t), want, target, f"skewed={skewed}")
+
+
+@pytest.mark.parametrize("target", TARGETS)
 def test_residual_after_every_layer_run(target):
     W = O.random_weights(FULL, seed=7)
     t = toks(17, seed=2)
