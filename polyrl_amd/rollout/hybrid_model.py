@@ -395,19 +395,27 @@ class RoutedMoE(_Part):
     def experts_large(self, h, idx):
         """Rows sorted by expert on the device, one vendor product pair per
         live expert (prompt-sized or fp32 batches); one host sync for the
-        row counts."""
+        row counts.  Each expert's products run over its rows rounded up to
+        a multiple of 64 (256 from 512 rows on), reading on into the next
+        expert's rows of the sorted copy: the vendor library then sees a
+        handful of shapes instead of a new one per call (a new shape costs
+        more on the host than the product takes on the GPU).  The surplus
+        rows' results are dropped."""
         N, top = idx.shape
+        S, W = N * top, h.shape[1]
         flat = idx.reshape(-1)
         order = torch.argsort(flat, stable=True)     # identity slots last
         counts = torch.bincount(flat, minlength=self.E + 1)[:self.E].tolist()
-        xs = h.index_select(0, order // top)
-        ys_sorted = torch.empty(N * top, h.shape[1], device=h.device,
-                                dtype=h.dtype)
+        xs = h.new_zeros(S + 256, W)
+        torch.index_select(h, 0, order // top, out=xs[:S])
+        ys_sorted = torch.empty(S, W, device=h.device, dtype=h.dtype)
         o = 0
         for e, c in enumerate(counts):
             if c:
-                act = seq.gelu_erf(_mm(xs[o:o + c], self.w_up[e]))
-                ys_sorted[o:o + c] = _mm(act, self.w_down[e])
+                step = 64 if c < 512 else 256
+                cp = -(-c // step) * step
+                act = seq.gelu_erf(_mm(xs[o:o + cp], self.w_up[e]))
+                ys_sorted[o:o + c] = _mm(act, self.w_down[e])[:c]
                 o += c
         ys = torch.empty_like(ys_sorted)
         ys[order] = ys_sorted           # identity rows stay unread
