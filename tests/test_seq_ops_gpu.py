@@ -349,6 +349,9 @@ def test_gqa_prepare_store(dt, H, G, D, Dv, half, norm, own_v):
     (2, 2, 128, 128, 33, 4, False, False, [70, 1], [10, 200]),
     (8, 2, 32, 96, 20, 0, True, False, [64, 1, 9], [0, 19, 64]),
     (3, 3, 200, 72, 5, 1, False, True, [6, 2], [0, 9]),
+    (4, 2, 64, 64, 16, 70, False, True, [100, 1, 40], [50, 300, 0]),
+    (2, 1, 40, 24, 200, 0, True, False, [130, 1, 70], [170, 450, 0]),
+    (4, 4, 96, 96, 40, 33, False, False, [1, 1, 1], [0, 31, 200]),
 ])
 def test_gqa_window_attention(dt, H, G, D, Dv, window, keep, bias, gate,
                               lens, starts):
